@@ -1,0 +1,207 @@
+// Calibration, page encoder and page decoder kernels + their extern "C" entry points.
+//   exponent_hist / bases_from_hist   /root/reference/gaac/codec.py:70-84
+//   encode_tiles / compact            /root/reference/gaac/encoder.py:16-76, 94-109
+//   row_offsets                       /root/reference/gaac/codec.py:221-225
+//   decode_tiles                      /root/reference/gaac/codec.py:186-218
+#include "gaac_tile.h"
+#include "gaac_capi.h"
+#include "../../include/gaac_hip.h"
+
+namespace gaac {
+
+char* last_error_buffer() { static thread_local char buf[512] = {0}; return buf; }
+
+// ---------------------------------------------------------------------------------------------------- calibration
+constexpr int HIST_CH = 32;     // channels per block (32 x 256 x 4 B = 32 KiB of LDS)
+__global__ void __launch_bounds__(256) k_exponent_hist(const u16* __restrict__ x, long n_tok, int n_kv, int chunk,
+                                                       unsigned long long* __restrict__ hist) {
+  __shared__ u32 h[HIST_CH * 256];
+  const int tid = threadIdx.x, c0 = blockIdx.x * HIST_CH;      // first of this block's channels in the n_kv*128 row
+  for (int i = tid; i < HIST_CH * 256; i += 256) h[i] = 0u;
+  __syncthreads();
+  const long t0 = (long)blockIdx.y * chunk, t1 = min(t0 + (long)chunk, n_tok);
+  const int c = tid & (HIST_CH - 1), sub = tid / HIST_CH;
+  const long row = (long)n_kv * D;
+  for (long t = t0 + sub; t < t1; t += 256 / HIST_CH) {
+    const u32 v = x[t * row + c0 + c];
+    atomicAdd(&h[c * 256 + ((v >> 7) & 0xFFu)], 1u);
+  }
+  __syncthreads();
+  for (int i = tid; i < HIST_CH * 256; i += 256)
+    if (h[i]) atomicAdd(&hist[(long)(c0 + (i >> 8)) * 256 + (i & 255)], (unsigned long long)h[i]);
+}
+
+__global__ void __launch_bounds__(128) k_bases_from_hist(const long long* __restrict__ hist, int rows,
+                                                         uint8_t* __restrict__ base3, uint8_t* __restrict__ base4) {
+  const int r = blockIdx.x * 128 + threadIdx.x;
+  if (r >= rows) return;
+  const long long* h = hist + (long)r * 256;
+  for (int pass = 0; pass < 2; ++pass) {          // densest 8-wide / 16-wide window, lowest start wins ties
+    const int w = pass ? 16 : 8;
+    long long s = 0;
+    for (int i = 0; i < w; ++i) s += h[i];
+    long long best = s; int arg = 0;
+    for (int st = 1; st + w <= 256; ++st) {
+      s += h[st + w - 1] - h[st - 1];
+      if (s > best) { best = s; arg = st; }
+    }
+    (pass ? base4 : base3)[r] = (uint8_t)arg;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------- page encoder
+template <int KIND>
+__global__ void __launch_bounds__(64) k_encode_tiles(const u16* __restrict__ x, int S, int S_in, int S_pad, const uint8_t* __restrict__ base3,
+                                                     const uint8_t* __restrict__ base4, int n_kv, const int* __restrict__ bidx,
+                                                     uint8_t* __restrict__ sm, uint8_t* __restrict__ cd, int* __restrict__ flags,
+                                                     uint8_t* __restrict__ esc_slots, int* __restrict__ tile_bytes, int ntiles) {
+  __shared__ EncodeLds L;
+  const int tile = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int brow = bidx ? bidx[h] : h % n_kv;
+  const int nvalid = min(T, S - tile * T);
+  stage_rows(L, x + ((long)h * S_in + (long)tile * T) * D, D, nvalid, lane);
+  stage_bases(L, base3 + (long)brow * D, base4 + (long)brow * D, lane);
+  __syncthreads();
+  const long row0 = (long)h * S_pad + (long)tile * T;
+  const int total = encode_staged_tile<KIND>(L, nvalid, lane, sm + row0 * D, cd + row0 * CB, flags + row0,
+                                             esc_slots + ((long)h * ntiles + tile) * TILE_MAX_ESC);
+  if (lane == 0) tile_bytes[(long)h * ntiles + tile] = total;
+}
+
+__global__ void __launch_bounds__(64) k_compact(const uint8_t* __restrict__ esc_slots, const int* __restrict__ tile_bytes,
+                                                const int* __restrict__ tile_off, const int* __restrict__ head_start,
+                                                uint8_t* __restrict__ ovf, int ntiles) {
+  const int tile = blockIdx.x, h = blockIdx.y;
+  const long i = (long)h * ntiles + tile;
+  const int n = tile_bytes[i];
+  const uint8_t* src = esc_slots + i * TILE_MAX_ESC;
+  uint8_t* dst = ovf + head_start[h] + tile_off[i];
+  for (int k = threadIdx.x; k < n; k += 64) dst[k] = src[k];
+}
+
+__global__ void __launch_bounds__(256) k_row_offsets(const int* __restrict__ flags, int S, int S_pad, int* __restrict__ out) {
+  __shared__ int sh[256];
+  __shared__ int carry;
+  const int h = blockIdx.x, tid = threadIdx.x;
+  if (tid == 0) carry = 0;
+  __syncthreads();
+  for (int base = 0; base < S; base += 256) {
+    const int s = base + tid;
+    const int rb = s < S ? esc_bytes((u32)flags[(long)h * S_pad + s]) : 0;
+    sh[tid] = rb;
+    __syncthreads();
+    for (int o = 1; o < 256; o <<= 1) {
+      int v = tid >= o ? sh[tid - o] : 0;
+      __syncthreads();
+      sh[tid] += v;
+      __syncthreads();
+    }
+    const int c = carry;
+    if (s < S) out[(long)h * S + s] = c + sh[tid] - rb;
+    __syncthreads();
+    if (tid == 255) carry = c + sh[255];
+    __syncthreads();
+  }
+}
+
+// ---------------------------------------------------------------------------------------------------- page decoder
+template <int KIND>
+__global__ void __launch_bounds__(64) k_decode_tiles(const uint8_t* __restrict__ sm, const uint8_t* __restrict__ cd, const int* __restrict__ flags,
+                                                     const int* __restrict__ tile_off, const uint8_t* __restrict__ ovf,
+                                                     const int* __restrict__ head_start, const uint8_t* __restrict__ base3,
+                                                     const uint8_t* __restrict__ base4, int n_kv, const int* __restrict__ bidx,
+                                                     int S, int S_pad, u16* __restrict__ out, long out_head_stride, long out_row_stride) {
+  const int tile = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, a = lane & 15, q = lane >> 4;
+  const int brow = bidx ? bidx[h] : h % n_kv;
+  const long row0 = (long)h * S_pad + (long)tile * T;
+  Payload P;
+  load_payload(sm + row0 * D, cd + row0 * CB, lane, P);
+  const u32 tag_word = (tile * T + a < S) ? (u32)flags[row0 + a] : 0u;
+  UnitMeta M;
+  tile_unit_meta<KIND>(tag_word, lane, M);
+  const uint8_t* esc = ovf + head_start[h] + tile_off[(long)h * (S_pad / T) + tile];
+  u32 b3w[4], b4w[4];
+  if (KIND == KIND_V) { load_base_words<KIND>(base3 + (long)brow * D, a, b3w); load_base_words<KIND>(base4 + (long)brow * D, a, b4w); }
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int tok = unit_token<KIND>(a, q, u), grp = unit_group<KIND>(a, q, u);
+    if (KIND == KIND_K) { load_base_words<KIND>(base3 + (long)brow * D, grp, b3w); load_base_words<KIND>(base4 + (long)brow * D, grp, b4w); }
+    u32 slo, shi, w[4];
+    unit_sm(P, u, slo, shi);
+    const u32 eb = M.tag[u] == 1u ? (u32)esc[M.pos[u]] : 0u;
+    decode_unit(slo, shi, unit_code_word(P.c0, P.c1, P.c2, u), M.tag[u], eb, esc + M.pos[u], b3w, b4w, w);
+    if (tile * T + tok < S) {
+      u16* o = out + (long)h * out_head_stride + (long)(tile * T + tok) * out_row_stride;
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        o[chan_of<KIND>(8 * grp + p)] = (u16)(w[p] & 0xFFFFu);
+        o[chan_of<KIND>(8 * grp + p + 4)] = (u16)(w[p] >> 16);
+      }
+    }
+  }
+}
+
+}  // namespace gaac
+
+using namespace gaac;
+
+extern "C" {
+
+const char* gaac_last_error(void) { return last_error_buffer(); }
+
+int gaac_exponent_hist(const void* x, long n_tokens, int n_kv, long long* hist, void* stream) {
+  GAAC_REQUIRE(x && hist && n_kv > 0 && n_tokens >= 0, "gaac_exponent_hist: bad arguments");
+  if (n_tokens == 0) return 0;
+  int nchunk = (int)min((n_tokens + 2047) / 2048, 256L);
+  int chunk = (int)((n_tokens + nchunk - 1) / nchunk);
+  hipLaunchKernelGGL(k_exponent_hist, dim3(n_kv * D / HIST_CH, nchunk), dim3(256), 0, (hipStream_t)stream,
+                     (const u16*)x, n_tokens, n_kv, chunk, (unsigned long long*)hist);
+  return launch_status("gaac_exponent_hist");
+}
+
+int gaac_bases_from_hist(const long long* hist, int rows, uint8_t* base3, uint8_t* base4, void* stream) {
+  GAAC_REQUIRE(hist && base3 && base4 && rows > 0, "gaac_bases_from_hist: bad arguments");
+  hipLaunchKernelGGL(k_bases_from_hist, dim3((rows + 127) / 128), dim3(128), 0, (hipStream_t)stream, hist, rows, base3, base4);
+  return launch_status("gaac_bases_from_hist");
+}
+
+int gaac_encode_tiles(int kind, const void* x, int H, int S, int S_in, int S_pad, const uint8_t* base3, const uint8_t* base4,
+                      int n_kv, const int* bidx, uint8_t* sm, uint8_t* codes, int* flags, uint8_t* esc_slots, int* tile_bytes,
+                      void* stream) {
+  GAAC_REQUIRE(kind == 0 || kind == 1, "gaac_encode_tiles: kind must be 0 (k) or 1 (v)");
+  GAAC_REQUIRE(x && base3 && base4 && sm && codes && flags && esc_slots && tile_bytes, "gaac_encode_tiles: null pointer");
+  GAAC_REQUIRE(H > 0 && S > 0 && S_in >= S && S_pad >= (S + T - 1) / T * T && S_pad % T == 0 && n_kv > 0,
+               "gaac_encode_tiles: bad sizes H=%d S=%d S_in=%d S_pad=%d n_kv=%d", H, S, S_in, S_pad, n_kv);
+  const int ntiles = (S + T - 1) / T;
+  dim3 grid(ntiles, H);
+  if (kind == 0) hipLaunchKernelGGL(k_encode_tiles<KIND_K>, grid, dim3(64), 0, (hipStream_t)stream, (const u16*)x, S, S_in, S_pad, base3, base4, n_kv, bidx, sm, codes, flags, esc_slots, tile_bytes, ntiles);
+  else hipLaunchKernelGGL(k_encode_tiles<KIND_V>, grid, dim3(64), 0, (hipStream_t)stream, (const u16*)x, S, S_in, S_pad, base3, base4, n_kv, bidx, sm, codes, flags, esc_slots, tile_bytes, ntiles);
+  return launch_status("gaac_encode_tiles");
+}
+
+int gaac_compact(const uint8_t* esc_slots, const int* tile_bytes, const int* tile_off, const int* head_start, uint8_t* ovf,
+                 int H, int ntiles, void* stream) {
+  GAAC_REQUIRE(esc_slots && tile_bytes && tile_off && head_start && ovf && H > 0 && ntiles > 0, "gaac_compact: bad arguments");
+  hipLaunchKernelGGL(k_compact, dim3(ntiles, H), dim3(64), 0, (hipStream_t)stream, esc_slots, tile_bytes, tile_off, head_start, ovf, ntiles);
+  return launch_status("gaac_compact");
+}
+
+int gaac_row_offsets(const int* flags, int H, int S, int S_pad, int* out, void* stream) {
+  GAAC_REQUIRE(flags && out && H > 0 && S > 0 && S_pad >= S, "gaac_row_offsets: bad arguments");
+  hipLaunchKernelGGL(k_row_offsets, dim3(H), dim3(256), 0, (hipStream_t)stream, flags, S, S_pad, out);
+  return launch_status("gaac_row_offsets");
+}
+
+int gaac_decode_tiles(int kind, const uint8_t* sm, const uint8_t* codes, const int* flags, const int* tile_off, const uint8_t* ovf,
+                      const int* head_start, const uint8_t* base3, const uint8_t* base4, int n_kv, const int* bidx, int H, int S,
+                      int S_pad, void* out, long out_head_stride, long out_row_stride, void* stream) {
+  GAAC_REQUIRE(kind == 0 || kind == 1, "gaac_decode_tiles: kind must be 0 (k) or 1 (v)");
+  GAAC_REQUIRE(sm && codes && flags && tile_off && ovf && head_start && base3 && base4 && out, "gaac_decode_tiles: null pointer");
+  GAAC_REQUIRE(H > 0 && S > 0 && S_pad >= (S + T - 1) / T * T && S_pad % T == 0 && n_kv > 0, "gaac_decode_tiles: bad sizes");
+  dim3 grid((S + T - 1) / T, H);
+  if (kind == 0) hipLaunchKernelGGL(k_decode_tiles<KIND_K>, grid, dim3(64), 0, (hipStream_t)stream, sm, codes, flags, tile_off, ovf, head_start, base3, base4, n_kv, bidx, S, S_pad, (u16*)out, out_head_stride, out_row_stride);
+  else hipLaunchKernelGGL(k_decode_tiles<KIND_V>, grid, dim3(64), 0, (hipStream_t)stream, sm, codes, flags, tile_off, ovf, head_start, base3, base4, n_kv, bidx, S, S_pad, (u16*)out, out_head_stride, out_row_stride);
+  return launch_status("gaac_decode_tiles");
+}
+
+}  // extern "C"

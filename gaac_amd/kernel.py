@@ -1,0 +1,65 @@
+"""Fused decode attention over the compressed KV on MI355X.  Public surface of /root/reference/gaac/kernel.py:332-359.
+
+attention() launches the split-K kernel (one block per (batch row, kv head, split), MFMA score and output products on
+K/V decoded in registers, optional raw-BF16 tail as one more block row) and the merge kernel, on the current stream,
+with no host synchronization.  Cache heads are addressed through a slot map exactly as in the reference: batch row b
+reads cache head SLOT[b]*n_kv + kvh, SLOT[b] < 0 = padded row (output 0)."""
+from __future__ import annotations
+import torch
+from . import _lib
+
+D = 128
+GMAX = 16
+MAX_SPLITS = 1023
+
+
+def _ext():
+    """The loaded native library (raises if it is not built)."""
+    return _lib.load()
+
+
+def choose_nsplit(B: int, n_kv: int, S: int, target_ctas: int = 512, min_tok: int = 256, cap: int = 256) -> int:
+    """Splits per (row, kv head): about 2 four-wave blocks per CU of the 256-CU MI355X (the reference targets 96 CTAs
+    for a 48-SM part, kernel.py:340-342), at least min_tok tokens per split."""
+    return min(max(1, target_ctas // (B * n_kv)), max(1, S // min_tok), cap)
+
+
+def attn_launch(K, V, q2d, slots, n_q, n_kv, SL, S_pad, scale, nsplit, kt=None, vt=None, TL=None, TCAP=0):
+    """K, V: objects with sm, codes, flags, tile_off, ovf, head_start|ovf_head_start, base3, base4 (a Page or a cache store).
+    q2d: [B*n_q, D] bf16 contiguous.  Returns [B*n_q, D] bf16."""
+    G = n_q // max(1, n_kv)
+    if not (1 <= G <= GMAX and G * n_kv == n_q):
+        raise RuntimeError(f"GQA group size must be 1..{GMAX}")
+    if q2d.shape[-1] != D:
+        raise RuntimeError("head_dim must be 128")
+    B = slots.shape[0]
+    dev = q2d.device
+    has_tail = kt is not None and kt.numel() > 0
+    nslot = nsplit + (1 if has_tail else 0)
+    out = torch.empty(B * n_q, D, dtype=q2d.dtype, device=dev)
+    pm = torch.empty(B * n_q * nslot, dtype=torch.float32, device=dev)
+    pl = torch.empty(B * n_q * nslot, dtype=torch.float32, device=dev)
+    pa = torch.empty(B * n_q * nslot * D, dtype=torch.float32, device=dev)
+    hs = lambda st: getattr(st, "head_start", None) if hasattr(st, "head_start") else st.ovf_head_start
+    p = _lib.ptr
+    _lib.call("gaac_attn_launch",
+              p(K.sm), p(K.codes), p(K.flags), p(K.tile_off), p(K.ovf), p(hs(K)), p(K.base3), p(K.base4),
+              p(V.sm), p(V.codes), p(V.flags), p(V.tile_off), p(V.ovf), p(hs(V)), p(V.base3), p(V.base4),
+              p(q2d), p(slots), B, n_q, n_kv, p(SL), S_pad, float(scale), nsplit, K.base3.shape[0],
+              p(kt) if has_tail else None, p(vt) if has_tail else None, p(TL) if has_tail else None, TCAP if has_tail else 0,
+              p(pm), p(pl), p(pa), p(out), _lib.stream())
+    return out
+
+
+def attention(q, kp, vp, scale=None, nsplit=None):
+    """Decode attention over two Pages (kinds 'k' / 'v', H = B*n_kv heads of equal length).
+    q: [B, n_q, D] bf16 (one query token per sequence) -> [B, n_q, D] bf16."""
+    B, n_q, Dq = q.shape
+    n_kv = kp.H // B
+    dev = q.device
+    if nsplit is None: nsplit = choose_nsplit(B, n_kv, kp.S)
+    slots = torch.arange(B, dtype=torch.int32, device=dev)
+    SL = torch.full((kp.H,), kp.S, dtype=torch.int32, device=dev)
+    out = attn_launch(kp, vp, q.reshape(B * n_q, Dq).contiguous(), slots, n_q, n_kv, SL, kp.sm.shape[1] // D,
+                      scale if scale is not None else Dq ** -0.5, nsplit)
+    return out.view(B, n_q, Dq)

@@ -1,0 +1,69 @@
+/* C-ABI of libgaac_hip.so: the MI355X (gfx950) kernels behind gaac_amd.{codec,encoder,kernel,kv_cache,paged}.
+ *
+ * Conventions for every entry point:
+ *   - all pointers are DEVICE pointers (plain, no framework types); `stream` is a hipStream_t passed as void*;
+ *   - nothing is allocated, nothing synchronizes, all work is enqueued on `stream` (graph-capture safe);
+ *   - returns 0 on success, -1 for rejected arguments, a positive hipError_t for a failed launch; the message
+ *     of the last failure on the calling thread is returned by gaac_last_error().
+ *   - BF16 tensors are passed as void* (16-bit patterns); `kind` is 0 for K, 1 for V.
+ *
+ * Byte order inside a 16-token tile (sign/mantissa and code bytes) is the gfx950 MFMA operand order documented in
+ * gaac_amd/csrc/gaac_core.h; tag words, tile offsets and the escape stream have the reference's order.
+ * Citations are to the reference interface each entry point replaces.
+ */
+#ifndef GAAC_HIP_H
+#define GAAC_HIP_H
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* gaac_last_error(void);
+
+/* exponent_hist(x, n_kv), /root/reference/gaac/codec.py:80-84.  x: bf16 [n_tokens, n_kv, 128] token-major;
+ * hist: int64 [n_kv*128, 256], ACCUMULATED into (zero it first). */
+int gaac_exponent_hist(const void* x, long n_tokens, int n_kv, long long* hist, void* stream);
+
+/* bases_from_hist(hist, n_kv), /root/reference/gaac/codec.py:70-77.  rows = n_kv*128; base3/base4: uint8 [rows]. */
+int gaac_bases_from_hist(const long long* hist, int rows, uint8_t* base3, uint8_t* base4, void* stream);
+
+/* TileEncoder.encode_tiles, /root/reference/gaac/encoder.py:16-66, 94-102 (same math as Codec.encode, codec.py:133-184).
+ * x: bf16 [H, S_in, 128]; tiles 0..ceil(S/16)-1 of every head are written to sm [H, S_pad*128], codes [H, S_pad*48],
+ * flags [H, S_pad]; escape bytes of tile (h, t) go to esc_slots[(h*ntiles+t)*1280 ...]; tile_bytes: int32 [H, ntiles].
+ * Head h uses base row bidx[h] (bidx != NULL) or h % n_kv. */
+int gaac_encode_tiles(int kind, const void* x, int H, int S, int S_in, int S_pad, const uint8_t* base3, const uint8_t* base4,
+                      int n_kv, const int* bidx, uint8_t* sm, uint8_t* codes, int* flags, uint8_t* esc_slots, int* tile_bytes,
+                      void* stream);
+
+/* TileEncoder.compact, /root/reference/gaac/encoder.py:69-76, 104-109: copies tile (h, t)'s tile_bytes[h, t] escape bytes
+ * from its 1280-byte slot to ovf + head_start[h] + tile_off[h, t]. */
+int gaac_compact(const uint8_t* esc_slots, const int* tile_bytes, const int* tile_off, const int* head_start, uint8_t* ovf,
+                 int H, int ntiles, void* stream);
+
+/* row_offsets(flags, S), /root/reference/gaac/codec.py:221-225.  flags: int32 [H, S_pad]; out: int32 [H, S]. */
+int gaac_row_offsets(const int* flags, int H, int S, int S_pad, int* out, void* stream);
+
+/* Codec.decode, /root/reference/gaac/codec.py:186-218.  Page fields as in the reference's Page dataclass
+ * (codec.py:87-102) with tile_off [H, S_pad/16]; out: bf16, element (h, s, c) at out[h*out_head_stride + s*out_row_stride + c]. */
+int gaac_decode_tiles(int kind, const uint8_t* sm, const uint8_t* codes, const int* flags, const int* tile_off, const uint8_t* ovf,
+                      const int* head_start, const uint8_t* base3, const uint8_t* base4, int n_kv, const int* bidx, int H, int S,
+                      int S_pad, void* out, long out_head_stride, long out_row_stride, void* stream);
+
+/* gaac_attn_launch, /root/reference/gaac/kernel.py:296-326 (kernels :48-294).  Same 16 store tensors, q [B*n_q, 128] bf16,
+ * slot map [B] (slot < 0 = padded row, output 0), SL [cache heads] compressed tokens per head, S_pad = token stride of a
+ * head, nsplit, and the optional raw tail kt/vt [cache heads, TCAP, 128] bf16 with lengths TL (kt == NULL: no tail).
+ * NB = rows of the base tables (n_kv, or the number of cache heads for per-sequence bases).
+ * Differences from the reference entry: the caller passes the partial buffers pm, pl [B*n_q*NSLOT] and
+ * pa [B*n_q*NSLOT*128] (fp32, NSLOT = nsplit + (kt != NULL)) and `out` [B*n_q, 128] bf16 instead of having them
+ * allocated inside; GQA group sizes 1..16 are accepted (reference: 1..8). */
+int gaac_attn_launch(
+    const uint8_t* smk, const uint8_t* ck, const int* fk, const int* tok, const uint8_t* ovk, const int* ohsk, const uint8_t* b3k, const uint8_t* b4k,
+    const uint8_t* smv, const uint8_t* cv, const int* fv, const int* tov, const uint8_t* ovv, const int* ohsv, const uint8_t* b3v, const uint8_t* b4v,
+    const void* q, const int* slot, int B, int n_q, int n_kv, const int* SL, int S_pad, float scale, int nsplit, int NB,
+    const void* kt, const void* vt, const int* TL, int TCAP,
+    float* pm, float* pl, float* pa, void* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

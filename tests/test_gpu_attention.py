@@ -1,0 +1,102 @@
+"""GPU parity of the fused decode attention against the oracle's fp32 attention over the DECODED K/V.
+Mirrors /root/reference/tests/test_kernel.py:6-19 (same shapes, same tolerance 2e-2*max|ref| + 1e-3) and adds the
+stated bar max-abs <= 1e-2 / mean-abs <= 1e-3 on N(0,1)-scale data, split-count independence and special cases."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gaac_oracle as O
+from common import kv_like16, to_bf16, to_u16, randn_bf16
+from gpu_util import require_gpu
+
+pytestmark = pytest.mark.gpu
+SCALE = 128 ** -0.5
+
+
+def _pages(B, n_kv, S, dev, seed=3):
+    from gaac_amd import Codec, TileEncoder
+    k16, v16 = kv_like16(B * n_kv, S, seed=seed), kv_like16(B * n_kv, S, seed=seed + 1)
+    k, v = to_bf16(k16, dev), to_bf16(v16, dev)
+    ck, cv = Codec(n_kv).calibrate(k), Codec(n_kv).calibrate(v)
+    return k16, v16, TileEncoder("k").encode(ck, k), TileEncoder("v").encode(cv, v)
+
+
+def _ref(q16, k16, v16, B, n_kv):
+    out = []
+    for b in range(B):
+        kb = k16[b * n_kv:(b + 1) * n_kv].transpose(1, 0, 2); vb = v16[b * n_kv:(b + 1) * n_kv].transpose(1, 0, 2)
+        out.append(O.ref_attention(q16[b], kb, vb, SCALE))
+    return np.stack(out)
+
+
+@pytest.mark.parametrize("B,n_kv,G", [(1, 8, 4), (2, 4, 8), (3, 2, 1), (1, 8, 2), (1, 4, 6), (1, 2, 16)])
+@pytest.mark.parametrize("S", [16, 333, 4096])
+def test_attention_matches_reference(B, n_kv, G, S):
+    dev = require_gpu()
+    from gaac_amd import attention
+    k16, v16, kp, vp = _pages(B, n_kv, S, dev)
+    q16 = randn_bf16((B, n_kv * G, 128), seed=7, scale=0.1)
+    out = attention(to_bf16(q16, dev), kp, vp, SCALE)
+    assert out.shape == (B, n_kv * G, 128) and out.dtype == torch.bfloat16
+    got = O.bf16_to_f32(to_u16(out)); ref = _ref(q16, k16, v16, B, n_kv)
+    for b in range(B):
+        err = np.abs(got[b] - ref[b]).max(); mag = np.abs(ref[b]).max()
+        assert err <= 2e-2 * mag + 1e-3, (b, err, mag)
+
+
+def test_result_does_not_depend_on_the_split_count():
+    dev = require_gpu()
+    from gaac_amd import attention
+    k16, v16, kp, vp = _pages(1, 4, 2000, dev, seed=11)
+    q = to_bf16(randn_bf16((1, 16, 128), seed=8, scale=0.5), dev)
+    outs = [O.bf16_to_f32(to_u16(attention(q, kp, vp, SCALE, nsplit=n))) for n in (1, 2, 7, 32, 125, 300)]
+    for o in outs[1:]:
+        assert np.abs(o - outs[0]).max() <= 2 ** -7 * np.abs(outs[0]).max()
+
+
+def test_stated_tolerance_on_unit_scale_data():
+    """max-abs <= 1e-2 and mean-abs <= 1e-3 against decompress + fp32 softmax attention, q ~ N(0,1)."""
+    dev = require_gpu()
+    from gaac_amd import attention, Codec, TileEncoder
+    n_kv, G, S = 8, 4, 8192
+    rng = np.random.default_rng(21)
+    k16 = O.f32_to_bf16_rne(rng.standard_normal((n_kv, S, 128)).astype(np.float32))
+    v16 = O.f32_to_bf16_rne(rng.standard_normal((n_kv, S, 128)).astype(np.float32))
+    k, v = to_bf16(k16, dev), to_bf16(v16, dev)
+    kp = TileEncoder("k").encode(Codec(n_kv).calibrate(k[:, :1024]), k)
+    vp = TileEncoder("v").encode(Codec(n_kv).calibrate(v[:, :1024]), v)
+    q16 = randn_bf16((1, n_kv * G, 128), seed=22)
+    got = O.bf16_to_f32(to_u16(attention(to_bf16(q16, dev), kp, vp, SCALE)))
+    ref = _ref(q16, k16, v16, 1, n_kv)
+    assert np.abs(got - ref).max() <= 1e-2 and np.abs(got - ref).mean() <= 1e-3
+
+
+def test_special_cases():
+    dev = require_gpu()
+    from gaac_amd import attention, Codec, TileEncoder
+    n_kv, G, S = 2, 4, 100
+    k16 = kv_like16(n_kv, S, seed=5)
+    row = randn_bf16((n_kv, 1, 128), seed=6)
+    v16 = np.ascontiguousarray(np.broadcast_to(row, (n_kv, S, 128)))          # all V rows equal -> output is that row
+    k, v = to_bf16(k16, dev), to_bf16(v16, dev)
+    kp, vp = TileEncoder("k").encode(Codec(n_kv).calibrate(k), k), TileEncoder("v").encode(Codec(n_kv).calibrate(v), v)
+    q16 = randn_bf16((1, n_kv * G, 128), seed=9, scale=0.2)
+    got = O.bf16_to_f32(to_u16(attention(to_bf16(q16, dev), kp, vp, SCALE)))[0]
+    want = np.repeat(O.bf16_to_f32(row[:, 0]), G, axis=0)
+    assert np.abs(got - want).max() <= 2 ** -7 * np.abs(want).max()
+    # q = 0 -> uniform weights -> mean of V
+    v16 = kv_like16(n_kv, S, seed=12, outliers=0.0)
+    v = to_bf16(v16, dev); vp = TileEncoder("v").encode(Codec(n_kv).calibrate(v), v)
+    got = O.bf16_to_f32(to_u16(attention(torch.zeros(1, n_kv * G, 128, dtype=torch.bfloat16, device=dev), kp, vp, SCALE)))[0]
+    want = np.repeat(O.bf16_to_f32(v16).mean(1), G, axis=0)
+    assert np.abs(got - want).max() <= 2e-2 * np.abs(want).max() + 1e-3
+
+
+def test_bad_arguments_raise():
+    dev = require_gpu()
+    from gaac_amd import attention
+    _, _, kp, vp = _pages(1, 2, 32, dev)
+    with pytest.raises(RuntimeError, match="group size"):
+        attention(torch.zeros(1, 2 * 17, 128, dtype=torch.bfloat16, device=dev), kp, vp, SCALE)
+    with pytest.raises(RuntimeError, match="head_dim"):
+        attention(torch.zeros(1, 4, 64, dtype=torch.bfloat16, device=dev), kp, vp, SCALE)
