@@ -313,20 +313,19 @@ __global__ void __launch_bounds__(128) k_attn_combine(const float* __restrict__ 
 
 using namespace gaac;
 
-extern "C" int gaac_attn_launch(
+static int attn_split_impl(
     const uint8_t* smk, const uint8_t* ck, const int* fk, const int* tok, const uint8_t* ovk, const int* ohsk, const uint8_t* b3k, const uint8_t* b4k,
     const uint8_t* smv, const uint8_t* cv, const int* fv, const int* tov, const uint8_t* ovv, const int* ohsv, const uint8_t* b3v, const uint8_t* b4v,
     const void* q, const int* slot, int B, int n_q, int n_kv, const int* SL, int S_pad, float scale, int nsplit, int NB,
-    const void* kt, const void* vt, const int* TL, int TCAP,
-    float* pm, float* pl, float* pa, void* out, void* stream) {
+    const void* kt, const void* vt, const int* TL, int TCAP, float* pm, float* pl, float* pa, void* stream) {
   GAAC_REQUIRE(n_kv > 0 && n_q > 0 && n_q % n_kv == 0 && n_q / n_kv >= 1 && n_q / n_kv <= GMAX, "GQA group size must be 1..%d (n_q=%d, n_kv=%d)", GMAX, n_q, n_kv);
-  GAAC_REQUIRE(smk && ck && fk && tok && ovk && ohsk && b3k && b4k && smv && cv && fv && tov && ovv && ohsv && b3v && b4v, "gaac_attn_launch: null store pointer");
-  GAAC_REQUIRE(q && slot && SL && pm && pl && pa && out, "gaac_attn_launch: null pointer");
-  GAAC_REQUIRE(B > 0 && S_pad > 0 && S_pad % T == 0 && NB > 0, "gaac_attn_launch: bad sizes B=%d S_pad=%d NB=%d", B, S_pad, NB);
+  GAAC_REQUIRE(smk && ck && fk && tok && ovk && ohsk && b3k && b4k && smv && cv && fv && tov && ovv && ohsv && b3v && b4v, "gaac_attn: null store pointer");
+  GAAC_REQUIRE(q && slot && SL && pm && pl && pa, "gaac_attn: null pointer");
+  GAAC_REQUIRE(B > 0 && S_pad > 0 && S_pad % T == 0 && NB > 0, "gaac_attn: bad sizes B=%d S_pad=%d NB=%d", B, S_pad, NB);
   const bool has_tail = kt != nullptr;
-  GAAC_REQUIRE(!has_tail || (vt && TL && TCAP >= 1 && TCAP <= T), "gaac_attn_launch: tail needs kt, vt, TL and 1 <= TCAP <= %d", T);
+  GAAC_REQUIRE(!has_tail || (vt && TL && TCAP >= 1 && TCAP <= T), "gaac_attn: tail needs kt, vt, TL and 1 <= TCAP <= %d", T);
   const int nslot = nsplit + (has_tail ? 1 : 0);
-  GAAC_REQUIRE(nsplit >= 1 && nslot <= MAX_SLOTS, "gaac_attn_launch: nsplit must be in 1..%d", MAX_SLOTS - 1);
+  GAAC_REQUIRE(nsplit >= 1 && nslot <= MAX_SLOTS, "gaac_attn: nsplit must be in 1..%d", MAX_SLOTS - 1);
   AttnArgs A;
   A.k = StoreView{smk, ck, fk, tok, ovk, ohsk, b3k, b4k};
   A.v = StoreView{smv, cv, fv, tov, ovv, ohsv, b3v, b4v};
@@ -335,8 +334,33 @@ extern "C" int gaac_attn_launch(
   A.n_kv = n_kv; A.n_q = n_q; A.G = n_q / n_kv; A.NB = NB;
   A.kt = (const u16*)kt; A.vt = (const u16*)vt; A.tl = TL; A.tcap = TCAP;
   hipLaunchKernelGGL(k_attn_split, dim3(B * n_kv, nslot), dim3(256), 0, (hipStream_t)stream, A);
-  int rc = launch_status("gaac_attn_launch(split)");
+  return launch_status("gaac_attn(split)");
+}
+
+extern "C" int gaac_attn_split(
+    const uint8_t* smk, const uint8_t* ck, const int* fk, const int* tok, const uint8_t* ovk, const int* ohsk, const uint8_t* b3k, const uint8_t* b4k,
+    const uint8_t* smv, const uint8_t* cv, const int* fv, const int* tov, const uint8_t* ovv, const int* ohsv, const uint8_t* b3v, const uint8_t* b4v,
+    const void* q, const int* slot, int B, int n_q, int n_kv, const int* SL, int S_pad, float scale, int nsplit, int NB,
+    const void* kt, const void* vt, const int* TL, int TCAP, float* pm, float* pl, float* pa, void* stream) {
+  return attn_split_impl(smk, ck, fk, tok, ovk, ohsk, b3k, b4k, smv, cv, fv, tov, ovv, ohsv, b3v, b4v, q, slot, B, n_q, n_kv, SL, S_pad,
+                         scale, nsplit, NB, kt, vt, TL, TCAP, pm, pl, pa, stream);
+}
+
+extern "C" int gaac_attn_combine(const float* pm, const float* pl, const float* pa, void* out, int n_rows, int nslot, void* stream) {
+  GAAC_REQUIRE(pm && pl && pa && out && n_rows > 0 && nslot >= 1 && nslot <= MAX_SLOTS, "gaac_attn_combine: bad arguments");
+  hipLaunchKernelGGL(k_attn_combine, dim3(n_rows), dim3(128), 0, (hipStream_t)stream, pm, pl, pa, (u16*)out, nslot);
+  return launch_status("gaac_attn(combine)");
+}
+
+extern "C" int gaac_attn_launch(
+    const uint8_t* smk, const uint8_t* ck, const int* fk, const int* tok, const uint8_t* ovk, const int* ohsk, const uint8_t* b3k, const uint8_t* b4k,
+    const uint8_t* smv, const uint8_t* cv, const int* fv, const int* tov, const uint8_t* ovv, const int* ohsv, const uint8_t* b3v, const uint8_t* b4v,
+    const void* q, const int* slot, int B, int n_q, int n_kv, const int* SL, int S_pad, float scale, int nsplit, int NB,
+    const void* kt, const void* vt, const int* TL, int TCAP,
+    float* pm, float* pl, float* pa, void* out, void* stream) {
+  GAAC_REQUIRE(out, "gaac_attn_launch: null output");
+  int rc = attn_split_impl(smk, ck, fk, tok, ovk, ohsk, b3k, b4k, smv, cv, fv, tov, ovv, ohsv, b3v, b4v, q, slot, B, n_q, n_kv, SL, S_pad,
+                           scale, nsplit, NB, kt, vt, TL, TCAP, pm, pl, pa, stream);
   if (rc) return rc;
-  hipLaunchKernelGGL(k_attn_combine, dim3(B * n_q), dim3(128), 0, (hipStream_t)stream, pm, pl, pa, (u16*)out, nslot);
-  return launch_status("gaac_attn_launch(combine)");
+  return gaac_attn_combine(pm, pl, pa, out, B * n_q, nsplit + (kt ? 1 : 0), stream);
 }

@@ -24,31 +24,49 @@ def choose_nsplit(B: int, n_kv: int, S: int, target_ctas: int = 512, min_tok: in
     return min(max(1, target_ctas // (B * n_kv)), max(1, S // min_tok), cap)
 
 
-def attn_launch(K, V, q2d, slots, n_q, n_kv, SL, S_pad, scale, nsplit, kt=None, vt=None, TL=None, TCAP=0):
+class AttnWorkspace:
+    """Output + split partials of one launch shape (fp32 m, l [rows*NSLOT] and acc [rows*NSLOT*D]; rows = B*n_q)."""
+    def __init__(self, rows: int, nslot: int, dtype, dev):
+        self.rows, self.nslot = rows, nslot
+        self.out = torch.empty(rows, D, dtype=dtype, device=dev)
+        self.pm = torch.empty(rows * nslot, dtype=torch.float32, device=dev)
+        self.pl = torch.empty(rows * nslot, dtype=torch.float32, device=dev)
+        self.pa = torch.empty(rows * nslot * D, dtype=torch.float32, device=dev)
+
+
+def _store_args(st):
+    p = _lib.ptr
+    hs = st.head_start if hasattr(st, "head_start") else st.ovf_head_start
+    return (p(st.sm), p(st.codes), p(st.flags), p(st.tile_off), p(st.ovf), p(hs), p(st.base3), p(st.base4))
+
+
+def attn_launch(K, V, q2d, slots, n_q, n_kv, SL, S_pad, scale, nsplit, kt=None, vt=None, TL=None, TCAP=0, ws=None, phase="both"):
     """K, V: objects with sm, codes, flags, tile_off, ovf, head_start|ovf_head_start, base3, base4 (a Page or a cache store).
-    q2d: [B*n_q, D] bf16 contiguous.  Returns [B*n_q, D] bf16."""
+    q2d: [B*n_q, D] bf16 contiguous.  Returns [B*n_q, D] bf16.  phase: "both" | "split" | "combine" (the halves of the launch)."""
     G = n_q // max(1, n_kv)
     if not (1 <= G <= GMAX and G * n_kv == n_q):
         raise RuntimeError(f"GQA group size must be 1..{GMAX}")
     if q2d.shape[-1] != D:
         raise RuntimeError("head_dim must be 128")
     B = slots.shape[0]
-    dev = q2d.device
     has_tail = kt is not None and kt.numel() > 0
     nslot = nsplit + (1 if has_tail else 0)
-    out = torch.empty(B * n_q, D, dtype=q2d.dtype, device=dev)
-    pm = torch.empty(B * n_q * nslot, dtype=torch.float32, device=dev)
-    pl = torch.empty(B * n_q * nslot, dtype=torch.float32, device=dev)
-    pa = torch.empty(B * n_q * nslot * D, dtype=torch.float32, device=dev)
-    hs = lambda st: getattr(st, "head_start", None) if hasattr(st, "head_start") else st.ovf_head_start
+    if ws is None:
+        ws = AttnWorkspace(B * n_q, nslot, q2d.dtype, q2d.device)
+    elif ws.rows != B * n_q or ws.nslot != nslot:
+        raise RuntimeError("attention workspace does not match the launch shape")
     p = _lib.ptr
-    _lib.call("gaac_attn_launch",
-              p(K.sm), p(K.codes), p(K.flags), p(K.tile_off), p(K.ovf), p(hs(K)), p(K.base3), p(K.base4),
-              p(V.sm), p(V.codes), p(V.flags), p(V.tile_off), p(V.ovf), p(hs(V)), p(V.base3), p(V.base4),
-              p(q2d), p(slots), B, n_q, n_kv, p(SL), S_pad, float(scale), nsplit, K.base3.shape[0],
-              p(kt) if has_tail else None, p(vt) if has_tail else None, p(TL) if has_tail else None, TCAP if has_tail else 0,
-              p(pm), p(pl), p(pa), p(out), _lib.stream())
-    return out
+    if phase == "combine":
+        _lib.call("gaac_attn_combine", p(ws.pm), p(ws.pl), p(ws.pa), p(ws.out), B * n_q, nslot, _lib.stream())
+        return ws.out
+    args = (*_store_args(K), *_store_args(V), p(q2d), p(slots), B, n_q, n_kv, p(SL), S_pad, float(scale), nsplit, K.base3.shape[0],
+            p(kt) if has_tail else None, p(vt) if has_tail else None, p(TL) if has_tail else None, TCAP if has_tail else 0,
+            p(ws.pm), p(ws.pl), p(ws.pa))
+    if phase == "split":
+        _lib.call("gaac_attn_split", *args, _lib.stream())
+    else:
+        _lib.call("gaac_attn_launch", *args, p(ws.out), _lib.stream())
+    return ws.out
 
 
 def attention(q, kp, vp, scale=None, nsplit=None):

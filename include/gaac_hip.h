@@ -63,6 +63,15 @@ int gaac_attn_launch(
     const void* kt, const void* vt, const int* TL, int TCAP,
     float* pm, float* pl, float* pa, void* out, void* stream);
 
+/* The two halves of gaac_attn_launch on their own (the split pass = gaac_attn + gaac_tail of kernel.py:48-279, the merge =
+ * gaac_combine of kernel.py:281-294), for callers that time or schedule them separately.  n_rows = B*n_q. */
+int gaac_attn_split(
+    const uint8_t* smk, const uint8_t* ck, const int* fk, const int* tok, const uint8_t* ovk, const int* ohsk, const uint8_t* b3k, const uint8_t* b4k,
+    const uint8_t* smv, const uint8_t* cv, const int* fv, const int* tov, const uint8_t* ovv, const int* ohsv, const uint8_t* b3v, const uint8_t* b4v,
+    const void* q, const int* slot, int B, int n_q, int n_kv, const int* SL, int S_pad, float scale, int nsplit, int NB,
+    const void* kt, const void* vt, const int* TL, int TCAP, float* pm, float* pl, float* pa, void* stream);
+int gaac_attn_combine(const float* pm, const float* pl, const float* pa, void* out, int n_rows, int nslot, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
