@@ -31,13 +31,6 @@ struct AttnArgs {
   const u16* kt; const u16* vt; const int* tl; int tcap;
 };
 
-struct TileRegs {                // one lane's view of a (K tile, V tile) pair
-  Payload k, v;
-  UnitMeta km, vm;
-  u32 keb[4], veb[4];
-  const uint8_t* kesc; const uint8_t* vesc;
-};
-
 __device__ __forceinline__ float bf16_bits_to_float(u32 h) { return __uint_as_float(h << 16); }
 __device__ __forceinline__ u32 pack_bf16x2(float lo, float hi) {
   typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
@@ -97,63 +90,185 @@ __device__ void tail_block(const AttnArgs& A, int b, int kvh, int ch, int slot) 
   }
 }
 
-// ---------------------------------------------------------------------------------------------------- tile loaders
-__device__ __forceinline__ void load_tags(const AttnArgs& A, long rowb, long tileb, int tile, int S, int a, u32& kfl, u32& vfl,
-                                          int& ktoff, int& vtoff) {
-  const int tok = tile * T + a;
-  kfl = tok < S ? (u32)A.k.flags[rowb + tok] : 0u;
-  vfl = tok < S ? (u32)A.v.flags[rowb + tok] : 0u;
-  ktoff = A.k.tile_off[tileb + tile];
-  vtoff = A.v.tile_off[tileb + tile];
+// ---------------------------------------------------------------------------------------------------- lookup tables
+// xlut[e]: the four exponent-field words carrying the 4th code bits of escape byte e (bit p -> element p, bit 4+p -> element p+4).
+// sel[m]:  v_perm selector that spreads a lane's packed 4-bit-group escape bytes to one byte per unit; m has bit 2u set when
+//          unit u owns an escape byte; byte u of the selector = index of that byte among the lane's bytes, or 0x0C (-> 0).
+struct AttnLds {
+  u32x4 xlut[256];
+  u32 sel[96];
+  float m[4][GMAX], l[4][GMAX];
+  float acc[4][GMAX][D];
+};
+__device__ __forceinline__ void build_luts(AttnLds& L, int tid) {
+  {
+    const u32 e = (u32)tid;
+    u32x4 w;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) w[p] = (((e >> p) & 1u) << 10) | (((e >> (4 + p)) & 1u) << 26);
+    L.xlut[tid] = w;
+  }
+  if (tid < 96) {
+    u32 selw = 0u, n = 0u;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const bool has = (tid >> (2 * u)) & 1;
+      selw |= (has ? n : 0x0Cu) << (8 * u);
+      n += has ? 1u : 0u;
+    }
+    L.sel[tid] = selw;
+  }
 }
-__device__ __forceinline__ void load_tile(const AttnArgs& A, long rowb, int tile, int lane, u32 kfl, u32 vfl,
-                                          const uint8_t* kesc, const uint8_t* vesc, TileRegs& R) {
-  const long row0 = rowb + (long)tile * T;
-  load_payload(A.k.sm + row0 * D, A.k.cd + row0 * CB, lane, R.k);
-  load_payload(A.v.sm + row0 * D, A.v.cd + row0 * CB, lane, R.v);
-  tile_unit_meta<KIND_K>(kfl, lane, R.km);
-  tile_unit_meta<KIND_V>(vfl, lane, R.vm);
-  R.kesc = kesc; R.vesc = vesc;
+
+// ---------------------------------------------------------------------------------------------------- tile loaders
+struct TileRegs {                // one lane's view of a (K tile, V tile) pair
+  Payload k, v;
+  u32 kf;                        // tag word of token a (K)
+  u32 kpos0;                     // offset of the lane's first K unit in the tile's escape bytes
+  u32x2 ke;                      // 8 escape bytes from kpos0 on
+  u32 vt8;                       // tags of the lane's 4 V units, 2 bits each
+  u32 vpos[4];                   // offsets of the 4 V units in the tile's escape bytes
+  u32x2 ve[4];                   // 8 escape bytes from each V unit's offset on
+};
+struct TagRegs { u32 kfl, vfl; u32 kto, vto; };
+
+struct Bases {                   // uniform (scalar) views of one cache head
+  const uint8_t* ksm; const uint8_t* kcd; const int* kfl; const int* kto; const uint8_t* kov;
+  const uint8_t* vsm; const uint8_t* vcd; const int* vfl; const int* vto; const uint8_t* vov;
+};
+
+__device__ __forceinline__ void load_tags(const Bases& B, int tile, int S, int a, TagRegs& Tg) {
+  const unsigned tok = (unsigned)(tile * T + a);
+  Tg.kfl = (u32)B.kfl[tok]; Tg.vfl = (u32)B.vfl[tok];
+  if ((int)tok >= S) { Tg.kfl = 0u; Tg.vfl = 0u; }
+  Tg.kto = (u32)B.kto[tile]; Tg.vto = (u32)B.vto[tile];
+}
+
+__device__ __forceinline__ void load_tile(const Bases& B, int tile, int lane, const TagRegs& Tg, const u32 (&bperm_addr)[4], TileRegs& R) {
+  const int a = lane & 15, q = lane >> 4;
+  load_payload(B.ksm + (size_t)tile * TILE_SM, B.kcd + (size_t)tile * TILE_CD, lane, R.k);
+  load_payload(B.vsm + (size_t)tile * TILE_SM, B.vcd + (size_t)tile * TILE_CD, lane, R.v);
+  // per-row escape bytes of K (low half) and V (high half), one scan for both
+  const u32 rb = (u32)esc_bytes(Tg.kfl) | ((u32)esc_bytes(Tg.vfl) << 16);
+  const u32 excl = row_scan16(rb) - rb;
+  R.kf = Tg.kfl;
+  R.kpos0 = (excl & 0xFFFFu) + (u32)esc_prefix(Tg.kfl, 8 * q);
+  R.ke = load_u32x2_unaligned(B.kov + Tg.kto + R.kpos0);
+  const u32 rov = excl >> 16;
+  R.vt8 = 0u;
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
-    R.keb[u] = R.km.tag[u] == 1u ? (u32)kesc[R.km.pos[u]] : 0u;
-    R.veb[u] = R.vm.tag[u] == 1u ? (u32)vesc[R.vm.pos[u]] : 0u;
+    const u32 f = (u32)__builtin_amdgcn_ds_bpermute((int)bperm_addr[u], (int)Tg.vfl);
+    const u32 ro = (u32)__builtin_amdgcn_ds_bpermute((int)bperm_addr[u], (int)rov);
+    R.vt8 |= ((f >> (2 * a)) & 3u) << (2 * u);
+    R.vpos[u] = ro + (u32)esc_prefix(f, 2 * a);
+    R.ve[u] = load_u32x2_unaligned(B.vov + Tg.vto + R.vpos[u]);
   }
 }
 
 // ---------------------------------------------------------------------------------------------------- one tile pair
-struct WaveState { f32x4 acc[8]; float m_run, l_run; };     // acc[i][r] = O[head a][group 4q+r, element i]
+struct WaveState { f32x4 acc[8]; float m_run, mu_run, l_run; };     // acc[i][r] = O[head a][group 4q+r, element i]
 
-__device__ __forceinline__ void consume_tile(const TileRegs& R, WaveState& st, int tile, int S, float scale_log2e, int a, int q,
+// unit decode with the escape contribution already expanded to exponent-field words x (see AttnLds::xlut)
+__device__ __forceinline__ void decode_unit_x(u32 slo, u32 shi, u32 g24, bool t0, const u32x4& x, const u32* __restrict__ b3w,
+                                              const u32* __restrict__ b4w, u32* __restrict__ out) {
+  const u32 cw = (g24 & 0xFFFu) | ((g24 << 4) & 0x0FFF0000u);
+  const u32 c0 = (cw << 7) & 0x03800380u, c1 = (cw << 4) & 0x03800380u, c2 = (cw << 1) & 0x03800380u, c3 = (cw >> 2) & 0x03800380u;
+  const u32 e0 = c0 + (t0 ? b3w[0] : b4w[0]) + x[0], e1 = c1 + (t0 ? b3w[1] : b4w[1]) + x[1];
+  const u32 e2 = c2 + (t0 ? b3w[2] : b4w[2]) + x[2], e3 = c3 + (t0 ? b3w[3] : b4w[3]) + x[3];
+  out[0] = (e0 & EXP_MASK2) | (__builtin_amdgcn_perm(shi, slo, 0x04040000u) & ~EXP_MASK2);
+  out[1] = (e1 & EXP_MASK2) | (__builtin_amdgcn_perm(shi, slo, 0x05050101u) & ~EXP_MASK2);
+  out[2] = (e2 & EXP_MASK2) | (__builtin_amdgcn_perm(shi, slo, 0x06060202u) & ~EXP_MASK2);
+  out[3] = (e3 & EXP_MASK2) | (__builtin_amdgcn_perm(shi, slo, 0x07070303u) & ~EXP_MASK2);
+}
+// raw group: 8 x 5 high exponent bits (40-bit little endian in lo/hi) as exponent-field words MINUS the 4-bit base words,
+// so that code + base4 + x reproduces code | hi5 << 3 exactly (32-bit arithmetic, the base cancels)
+__device__ __forceinline__ u32x4 raw_x_words(u32 lo, u32 hi, const u32* __restrict__ b4w) {
+  u32x4 x;
+  x[0] = (((lo) & 31u) << 10 | ((lo >> 20) & 31u) << 26) - b4w[0];
+  x[1] = (((lo >> 5) & 31u) << 10 | ((lo >> 25) & 31u) << 26) - b4w[1];
+  x[2] = (((lo >> 10) & 31u) << 10 | (__builtin_amdgcn_alignbit(hi, lo, 30) & 31u) << 26) - b4w[2];
+  x[3] = (((lo >> 15) & 31u) << 10 | ((hi >> 3) & 31u) << 26) - b4w[3];
+  return x;
+}
+
+__device__ __forceinline__ void consume_tile(const TileRegs& R, WaveState& st, AttnLds& L, const Bases& B,
+                                             u32 kto, u32 vto, int tile, int S, float scale_log2e, int a, int q,
                                              const u32x4 (&qf)[4], const u32 (&kb3)[4][4], const u32 (&kb4)[4][4],
                                              const u32 (&vb3)[4], const u32 (&vb4)[4]) {
+  // ---- K escapes: spread the lane's 4-bit-group bytes to units, expand through the table
+  const u32 ktag8 = __builtin_amdgcn_ubfe(R.kf, 8 * q, 8);
+  u32x4 x[4];
+  {
+    const u32 eb4 = __builtin_amdgcn_perm(0u, R.ke[0], L.sel[ktag8 & 0x55u]);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) x[u] = L.xlut[(eb4 >> (8 * u)) & 0xFFu];
+  }
+  if (__builtin_amdgcn_ballot_w64((ktag8 & 0xAAu) != 0u)) {      // some lane holds a raw group (rare per lane, common per tile)
+    if (ktag8 & 0xAAu) {                                          // redo every escaped unit of this lane at its true offset
+      u32 off = 0u;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const u32 t = (ktag8 >> (2 * u)) & 3u;
+        if (t) {
+          u32 lo, hi;
+          if (off + (u32)tag_size(t) <= 8u) {
+            const u64 v = ((u64)R.ke[0] | ((u64)R.ke[1] << 32)) >> (8u * off);
+            lo = (u32)v; hi = (u32)(v >> 32);
+          } else {
+            const u64 v = load_u64_unaligned(B.kov + kto + R.kpos0 + off);
+            lo = (u32)v; hi = (u32)(v >> 32);
+          }
+          x[u] = t == 1u ? L.xlut[lo & 0xFFu] : raw_x_words(lo, hi, kb4[u]);
+        }
+        off += (u32)tag_size(t);
+      }
+    }
+  }
   // ---- scores: S[tok 4q+r][head a]
   f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
     u32 slo, shi, w[4];
     unit_sm(R.k, u, slo, shi);
-    decode_unit(slo, shi, unit_code_word(R.k.c0, R.k.c1, R.k.c2, u), R.km.tag[u], R.keb[u], R.kesc + R.km.pos[u], kb3[u], kb4[u], w);
+    decode_unit_x(slo, shi, unit_code_word(R.k.c0, R.k.c1, R.k.c2, u), ((ktag8 >> (2 * u)) & 1u) == 0u, x[u], kb3[u], kb4[u], w);
     const u32x4 av = {w[0], w[1], w[2], w[3]};
     sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av), __builtin_bit_cast(bf16x8, qf[u]), sacc, 0, 0, 0);
   }
-  // ---- online softmax per head a over the tile's 16 tokens (4 in this lane, 4 quads)
+  // ---- V escapes (each unit has its own 8 bytes)
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const bool t0 = ((R.vt8 >> (2 * u)) & 1u) == 0u;
+    x[u] = L.xlut[t0 ? 0u : (R.ve[u][0] & 0xFFu)];
+  }
+  if (__builtin_amdgcn_ballot_w64((R.vt8 & 0xAAu) != 0u)) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (((R.vt8 >> (2 * u)) & 3u) == 3u) x[u] = raw_x_words(R.ve[u][0], R.ve[u][1], vb4);
+  }
+  // ---- online softmax per head a over the tile's 16 tokens (4 in this lane, 4 quads), base 2
   const int tok0 = tile * T + 4 * q;
   float s[4];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) s[r] = tok0 + r < S ? sacc[r] * scale_log2e : -INFINITY;
-  const float tmax = quad_rows_max(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
-  const float mn = fmaxf(st.m_run, tmax), mu = mn == -INFINITY ? 0.f : mn;
-  const float alpha = __builtin_amdgcn_exp2f(st.m_run - mu);
-  float p[4];
+  for (int r = 0; r < 4; ++r) s[r] = sacc[r] * scale_log2e;
+  const bool partial = tile * T + T > S;          // uniform: only the last tile of a sequence can be partly filled
+  if (partial) {
 #pragma unroll
-  for (int r = 0; r < 4; ++r) p[r] = __builtin_amdgcn_exp2f(s[r] - mu);
-  st.l_run = st.l_run * alpha + ((p[0] + p[1]) + (p[2] + p[3]));
-  st.m_run = mn;
-  if (__builtin_amdgcn_ballot_w64(alpha != 1.f)) {
+    for (int r = 0; r < 4; ++r) if (tok0 + r >= S) s[r] = -INFINITY;
+  }
+  const float tmax = quad_rows_max(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
+  if (__builtin_amdgcn_ballot_w64(tmax > st.m_run)) {             // the running maximum of some head grows (rare after the first tiles)
+    const float mn = fmaxf(st.m_run, tmax), mu = mn == -INFINITY ? 0.f : mn;
+    const float alpha = __builtin_amdgcn_exp2f(st.m_run - mu);
+    st.l_run *= alpha;
 #pragma unroll
     for (int i = 0; i < 8; ++i) st.acc[i] *= alpha;
+    st.m_run = mn; st.mu_run = mu;
   }
+  float p[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) p[r] = __builtin_amdgcn_exp2f(s[r] - st.mu_run);
+  st.l_run += (p[0] + p[1]) + (p[2] + p[3]);
   const u32x2 pw = {pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3])};
   const s16x4 pb = __builtin_bit_cast(s16x4, pw);
   // ---- values: decode the lane's 4 tokens of group a, regroup as token pairs per element, accumulate O^T
@@ -162,9 +277,9 @@ __device__ __forceinline__ void consume_tile(const TileRegs& R, WaveState& st, i
   for (int u = 0; u < 4; ++u) {
     u32 slo, shi;
     unit_sm(R.v, u, slo, shi);
-    decode_unit(slo, shi, unit_code_word(R.v.c0, R.v.c1, R.v.c2, u), R.vm.tag[u], R.veb[u], R.vesc + R.vm.pos[u], vb3, vb4, W[u]);
+    decode_unit_x(slo, shi, unit_code_word(R.v.c0, R.v.c1, R.v.c2, u), ((R.vt8 >> (2 * u)) & 1u) == 0u, x[u], vb3, vb4, W[u]);
   }
-  if (tile * T + T > S) {       // last, partly filled tile: rows beyond the sequence must not reach the product
+  if (partial) {                // rows beyond the sequence must not reach the product
 #pragma unroll
     for (int u = 0; u < 4; ++u)
       if (tok0 + u >= S) { W[u][0] = W[u][1] = W[u][2] = W[u][3] = 0u; }
@@ -180,10 +295,12 @@ __device__ __forceinline__ void consume_tile(const TileRegs& R, WaveState& st, i
 
 // ---------------------------------------------------------------------------------------------------- main kernel
 __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
+  __shared__ AttnLds L;
   const int bh = blockIdx.x, split = blockIdx.y, tid = threadIdx.x;
   const int b = bh / A.n_kv, kvh = bh % A.n_kv, G = A.G;
   const int slot = A.slot[b], ch = (slot < 0 ? 0 : slot) * A.n_kv + kvh;
   if (split == A.nsplit) { tail_block(A, b, kvh, ch, slot); return; }
+  build_luts(L, tid);
 
   const int S = slot < 0 ? 0 : A.sl[ch];
   const int ntiles = (S + T - 1) / T, chunk = (ntiles + A.nsplit - 1) / A.nsplit;
@@ -191,8 +308,9 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, a = lane & 15, q = lane >> 4;
   const long rowb = (long)ch * A.S_pad, tileb = (long)ch * (A.S_pad / T);
   const long qh0 = (long)b * A.n_q + (long)kvh * G;
-  const uint8_t* ovk = A.k.ovf + A.k.head_start[ch];
-  const uint8_t* ovv = A.v.ovf + A.v.head_start[ch];
+  Bases B;
+  B.ksm = A.k.sm + rowb * D; B.kcd = A.k.cd + rowb * CB; B.kfl = A.k.flags + rowb; B.kto = A.k.tile_off + tileb; B.kov = A.k.ovf + A.k.head_start[ch];
+  B.vsm = A.v.sm + rowb * D; B.vcd = A.v.cd + rowb * CB; B.vfl = A.v.flags + rowb; B.vto = A.v.tile_off + tileb; B.vov = A.v.ovf + A.v.head_start[ch];
 
   // Q as the B operand of the score product: lane (head a, quad q), product u covers group 4q+u in word order (e, e+4)
   u32x4 qf[4];
@@ -218,59 +336,73 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
   }
   load_base_words<KIND_V>(A.v.base3 + (long)brow * D, a, vb3);
   load_base_words<KIND_V>(A.v.base4 + (long)brow * D, a, vb4);
+  u32 bperm_addr[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) bperm_addr[u] = (u32)(4 * (4 * q + u));
+  __syncthreads();        // lookup tables are ready
 
   WaveState st;
 #pragma unroll
   for (int i = 0; i < 8; ++i) st.acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-  st.m_run = -INFINITY; st.l_run = 0.f;
+  st.m_run = -INFINITY; st.mu_run = 0.f; st.l_run = 0.f;
 
-  TileRegs R0, R1;                 // ping-pong: one is consumed while the other is being loaded
-  u32 kflN = 0u, vflN = 0u; int ktoN = 0, vtoN = 0;
-  int tile = tlo + wave;
-  if (tile < thi) {
-    u32 kf, vf; int kto, vto;
-    load_tags(A, rowb, tileb, tile, S, a, kf, vf, kto, vto);
-    if (tile + 4 < thi) load_tags(A, rowb, tileb, tile + 4, S, a, kflN, vflN, ktoN, vtoN);
-    load_tile(A, rowb, tile, lane, kf, vf, ovk + kto, ovv + vto, R0);
-  }
-  for (; tile < thi; tile += 8) {
-    if (tile + 4 < thi) {
-      load_tile(A, rowb, tile + 4, lane, kflN, vflN, ovk + ktoN, ovv + vtoN, R1);
-      if (tile + 8 < thi) load_tags(A, rowb, tileb, tile + 8, S, a, kflN, vflN, ktoN, vtoN);
+  // tiles of this wave: t(i) = tlo + wave + 4 i, i < n.  Ping-pong registers R0/R1; tag words are fetched one tile further
+  // ahead (index clamped to the wave's last tile, so that no load sits under a branch the consumer has to join).
+  const int t0 = tlo + wave;
+  const int n = t0 < thi ? (thi - t0 + 3) / 4 : 0;
+  if (n > 0) {
+    const int tlast = t0 + 4 * (n - 1);
+    TileRegs R0, R1;
+    TagRegs Tg, TgC0, TgC1;
+    load_tags(B, t0, S, a, Tg);
+    TgC0 = Tg;
+    load_tile(B, t0, lane, Tg, bperm_addr, R0);
+    load_tags(B, min(t0 + 4, tlast), S, a, Tg);
+    int i = 0;
+    for (; i + 2 < n; i += 2) {
+      const int t = t0 + 4 * i;
+      TgC1 = Tg;
+      load_tile(B, t + 4, lane, Tg, bperm_addr, R1);
+      load_tags(B, min(t + 8, tlast), S, a, Tg);
+      consume_tile(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+      TgC0 = Tg;
+      load_tile(B, t + 8, lane, Tg, bperm_addr, R0);
+      load_tags(B, min(t + 12, tlast), S, a, Tg);
+      consume_tile(R1, st, L, B, TgC1.kto, TgC1.vto, t + 4, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
     }
-    consume_tile(R0, st, tile, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
-    if (tile + 4 >= thi) break;
-    if (tile + 8 < thi) {
-      load_tile(A, rowb, tile + 8, lane, kflN, vflN, ovk + ktoN, ovv + vtoN, R0);
-      if (tile + 12 < thi) load_tags(A, rowb, tileb, tile + 12, S, a, kflN, vflN, ktoN, vtoN);
+    const int t = t0 + 4 * i;
+    if (n - i == 2) {
+      TgC1 = Tg;
+      load_tile(B, t + 4, lane, Tg, bperm_addr, R1);
+      consume_tile(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+      consume_tile(R1, st, L, B, TgC1.kto, TgC1.vto, t + 4, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+    } else {
+      consume_tile(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
     }
-    consume_tile(R1, st, tile + 4, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
   }
   float m_run = st.m_run, l_run = st.l_run;
   f32x4 (&acc)[8] = st.acc;
 
   // ---- merge the 4 waves of the block, write the split's partial
-  __shared__ float sh_m[4][GMAX], sh_l[4][GMAX];
-  __shared__ float sh_acc[4][GMAX][D];
   l_run = quad_rows_sum(l_run);
   if (a < G) {
-    if (q == 0) { sh_m[wave][a] = m_run; sh_l[wave][a] = l_run; }
+    if (q == 0) { L.m[wave][a] = m_run; L.l[wave][a] = l_run; }
 #pragma unroll
     for (int i = 0; i < 8; ++i)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) sh_acc[wave][a][chan_v(8 * (4 * q + r) + i)] = acc[i][r];
+      for (int r = 0; r < 4; ++r) L.acc[wave][a][chan_v(8 * (4 * q + r) + i)] = acc[i][r];
   }
   __syncthreads();
   const int d = tid & 127;
   for (int g = tid >> 7; g < G; g += 2) {
     float M = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) M = fmaxf(M, sh_m[w][g]);
+    for (int w = 0; w < 4; ++w) M = fmaxf(M, L.m[w][g]);
     float Lc = 0.f, Ac = 0.f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-      const float f = sh_m[w][g] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(sh_m[w][g] - M);
-      Lc += sh_l[w][g] * f; Ac += sh_acc[w][g][d] * f;
+      const float f = L.m[w][g] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(L.m[w][g] - M);
+      Lc += L.l[w][g] * f; Ac += L.acc[w][g][d] * f;
     }
     const long pidx = (qh0 + g) * A.nslot + split;
     if (d == 0) { A.pm[pidx] = M; A.pl[pidx] = Lc; }

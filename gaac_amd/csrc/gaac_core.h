@@ -160,6 +160,7 @@ __device__ __forceinline__ void unit_sm(const Payload& P, int u, u32& slo, u32& 
 }
 
 // unaligned little-endian loads from the escape stream (the stream is padded by 8 bytes at the end)
+__device__ __forceinline__ u32x2 load_u32x2_unaligned(const uint8_t* p) { u32x2 v; __builtin_memcpy(&v, p, 8); return v; }
 __device__ __forceinline__ u64 load_u64_unaligned(const uint8_t* p) {
   u32x2 v; __builtin_memcpy(&v, p, 8); return (u64)v[0] | ((u64)v[1] << 32);
 }
