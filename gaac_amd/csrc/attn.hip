@@ -90,46 +90,65 @@ __device__ void tail_block(const AttnArgs& A, int b, int kvh, int ch, int slot) 
   }
 }
 
-// ---------------------------------------------------------------------------------------------------- lookup tables
+// ---------------------------------------------------------------------------------------------------- block tables (LDS)
 // xlut[e]: the four exponent-field words carrying the 4th code bits of escape byte e (bit p -> element p, bit 4+p -> element p+4).
-// sel[m]:  v_perm selector that spreads a lane's packed 4-bit-group escape bytes to one byte per unit; m has bit 2u set when
-//          unit u owns an escape byte; byte u of the selector = index of that byte among the lane's bytes, or 0x0C (-> 0).
+// sel[t]:  v_perm selector that spreads a lane's 8 prefetched escape bytes to one byte per unit, indexed by the lane's four
+//          tags t (2 bits each): byte u = offset of unit u's escape byte when the unit is a 4-bit group (and the offset
+//          is < 8), else 0x0C (-> 0).
+// bw*:     exponent-base words [tier][group][p] of this block's kv head;  qw: the query words [head][group][p].
 struct AttnLds {
   u32x4 xlut[256];
-  u32 sel[96];
+  u32 sel[256];
+  u32x4 bwk[2][NG], bwv[2][NG];
+  u32x4 qw[GMAX][NG];
   float m[4][GMAX], l[4][GMAX];
   float acc[4][GMAX][D];
 };
-__device__ __forceinline__ void build_luts(AttnLds& L, int tid) {
+__device__ __forceinline__ void build_tables(AttnLds& L, int tid, const AttnArgs& A, int brow, long qh0) {
   {
     const u32 e = (u32)tid;
     u32x4 w;
 #pragma unroll
     for (int p = 0; p < 4; ++p) w[p] = (((e >> p) & 1u) << 10) | (((e >> (4 + p)) & 1u) << 26);
     L.xlut[tid] = w;
-  }
-  if (tid < 96) {
-    u32 selw = 0u, n = 0u;
+    u32 selw = 0u, off = 0u;
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      const bool has = (tid >> (2 * u)) & 1;
-      selw |= (has ? n : 0x0Cu) << (8 * u);
-      n += has ? 1u : 0u;
+      const u32 t = (e >> (2 * u)) & 3u;
+      selw |= ((t == 1u && off < 8u) ? off : 0x0Cu) << (8 * u);
+      off += (u32)tag_size(t);
     }
     L.sel[tid] = selw;
+  }
+  {   // one base word per thread: kind = tid >> 7, tier = (tid >> 6) & 1, group = (tid >> 2) & 15, p = tid & 3
+    const int kind = tid >> 7, tier = (tid >> 6) & 1, g = (tid >> 2) & 15, p = tid & 3;
+    const StoreView& st = kind ? A.v : A.k;
+    const uint8_t* row = (tier ? st.base4 : st.base3) + (long)brow * D;
+    const int c0 = kind ? chan_v(8 * g + p) : chan_k(8 * g + p), c1 = kind ? chan_v(8 * g + p + 4) : chan_k(8 * g + p + 4);
+    const u32 w = ((u32)row[c0] << 7) | ((u32)row[c1] << 23);
+    u32* dst = kind ? reinterpret_cast<u32*>(&L.bwv[tier][g]) : reinterpret_cast<u32*>(&L.bwk[tier][g]);
+    dst[p] = w;
+  }
+#pragma unroll
+  for (int k = 0; k < (GMAX * NG * 4) / 256; ++k) {      // query words: head = idx >> 6, group = (idx >> 2) & 15, p = idx & 3
+    const int idx = tid + 256 * k, h = idx >> 6, g = (idx >> 2) & 15, p = idx & 3;
+    u32 w = 0u;
+    if (h < A.G) {
+      const u16* qp = A.q + (qh0 + h) * D;
+      w = (u32)qp[chan_k(8 * g + p)] | ((u32)qp[chan_k(8 * g + p + 4)] << 16);
+    }
+    reinterpret_cast<u32*>(&L.qw[h][g])[p] = w;
   }
 }
 
 // ---------------------------------------------------------------------------------------------------- tile loaders
-struct TileRegs {                // one lane's view of a (K tile, V tile) pair
-  Payload k, v;
-  u32 kf;                        // tag word of token a (K)
-  u32 kpos0;                     // offset of the lane's first K unit in the tile's escape bytes
-  u32x2 ke;                      // 8 escape bytes from kpos0 on
-  u32 vt8;                       // tags of the lane's 4 V units, 2 bits each
-  u32 vpos[4];                   // offsets of the 4 V units in the tile's escape bytes
-  u32x2 ve[4];                   // 8 escape bytes from each V unit's offset on
+struct KindRegs {                // one lane's view of one tile (K or V)
+  Payload pay;
+  u32 f;                         // tag word of the lane's line
+  u32 pos0;                      // offset of the lane's first unit in the tile's escape bytes
+  u32x2 e;                       // the 8 escape bytes from pos0 on
 };
+struct TileRegs { KindRegs k, v; };
 struct TagRegs { u32 kfl, vfl; u32 kto, vto; };
 
 struct Bases {                   // uniform (scalar) views of one cache head
@@ -137,45 +156,37 @@ struct Bases {                   // uniform (scalar) views of one cache head
   const uint8_t* vsm; const uint8_t* vcd; const int* vfl; const int* vto; const uint8_t* vov;
 };
 
-__device__ __forceinline__ void load_tags(const Bases& B, int tile, int S, int a, TagRegs& Tg) {
-  const unsigned tok = (unsigned)(tile * T + a);
-  Tg.kfl = (u32)B.kfl[tok]; Tg.vfl = (u32)B.vfl[tok];
-  if ((int)tok >= S) { Tg.kfl = 0u; Tg.vfl = 0u; }
+__device__ __forceinline__ void load_tags(const Bases& B, int tile, int a, TagRegs& Tg) {
+  const unsigned w = (unsigned)(tile * T + a);
+  Tg.kfl = (u32)B.kfl[w]; Tg.vfl = (u32)B.vfl[w];
   Tg.kto = (u32)B.kto[tile]; Tg.vto = (u32)B.vto[tile];
 }
 
-__device__ __forceinline__ void load_tile(const Bases& B, int tile, int lane, const TagRegs& Tg, const u32 (&bperm_addr)[4], TileRegs& R) {
-  const int a = lane & 15, q = lane >> 4;
-  load_payload(B.ksm + (size_t)tile * TILE_SM, B.kcd + (size_t)tile * TILE_CD, lane, R.k);
-  load_payload(B.vsm + (size_t)tile * TILE_SM, B.vcd + (size_t)tile * TILE_CD, lane, R.v);
-  // per-row escape bytes of K (low half) and V (high half), one scan for both
+__device__ __forceinline__ void load_tile(const Bases& B, int tile, int lane, const TagRegs& Tg, TileRegs& R) {
+  const int q = lane >> 4;
+  load_payload(B.ksm + (size_t)tile * TILE_SM, B.kcd + (size_t)tile * TILE_CD, lane, R.k.pay);
+  load_payload(B.vsm + (size_t)tile * TILE_SM, B.vcd + (size_t)tile * TILE_CD, lane, R.v.pay);
+  // escape bytes per line of K (low half) and V (high half): one scan for both
   const u32 rb = (u32)esc_bytes(Tg.kfl) | ((u32)esc_bytes(Tg.vfl) << 16);
   const u32 excl = row_scan16(rb) - rb;
-  R.kf = Tg.kfl;
-  R.kpos0 = (excl & 0xFFFFu) + (u32)esc_prefix(Tg.kfl, 8 * q);
-  R.ke = load_u32x2_unaligned(B.kov + Tg.kto + R.kpos0);
-  const u32 rov = excl >> 16;
-  R.vt8 = 0u;
-#pragma unroll
-  for (int u = 0; u < 4; ++u) {
-    const u32 f = (u32)__builtin_amdgcn_ds_bpermute((int)bperm_addr[u], (int)Tg.vfl);
-    const u32 ro = (u32)__builtin_amdgcn_ds_bpermute((int)bperm_addr[u], (int)rov);
-    R.vt8 |= ((f >> (2 * a)) & 3u) << (2 * u);
-    R.vpos[u] = ro + (u32)esc_prefix(f, 2 * a);
-    R.ve[u] = load_u32x2_unaligned(B.vov + Tg.vto + R.vpos[u]);
-  }
+  R.k.f = Tg.kfl; R.v.f = Tg.vfl;
+  R.k.pos0 = (excl & 0xFFFFu) + (u32)esc_prefix(Tg.kfl, 8 * q);
+  R.v.pos0 = (excl >> 16) + (u32)esc_prefix(Tg.vfl, 8 * q);
+  R.k.e = load_u32x2_unaligned(B.kov + Tg.kto + R.k.pos0);
+  R.v.e = load_u32x2_unaligned(B.vov + Tg.vto + R.v.pos0);
 }
 
 // ---------------------------------------------------------------------------------------------------- one tile pair
-struct WaveState { f32x4 acc[8]; float m_run, mu_run, l_run; };     // acc[i][r] = O[head a][group 4q+r, element i]
+struct WaveState { f32x4 acc[8]; float m_run, mu_run, l_run; };     // acc[i][r] = O[head a][group 4q+r, element i]; m in raw score units
 
 // unit decode with the escape contribution already expanded to exponent-field words x (see AttnLds::xlut)
-__device__ __forceinline__ void decode_unit_x(u32 slo, u32 shi, u32 g24, bool t0, const u32x4& x, const u32* __restrict__ b3w,
-                                              const u32* __restrict__ b4w, u32* __restrict__ out) {
+__device__ __forceinline__ void decode_unit_x(u32 slo, u32 shi, u32 g24, u32 tmask, const u32x4& x, const u32x4& b3w, const u32x4& b4w,
+                                              u32* __restrict__ out) {
   const u32 cw = (g24 & 0xFFFu) | ((g24 << 4) & 0x0FFF0000u);
   const u32 c0 = (cw << 7) & 0x03800380u, c1 = (cw << 4) & 0x03800380u, c2 = (cw << 1) & 0x03800380u, c3 = (cw >> 2) & 0x03800380u;
-  const u32 e0 = c0 + (t0 ? b3w[0] : b4w[0]) + x[0], e1 = c1 + (t0 ? b3w[1] : b4w[1]) + x[1];
-  const u32 e2 = c2 + (t0 ? b3w[2] : b4w[2]) + x[2], e3 = c3 + (t0 ? b3w[3] : b4w[3]) + x[3];
+  // tmask = 0 for a 3-bit group (base3), ~0 otherwise (base4)
+  const u32 e0 = c0 + ((b4w[0] & tmask) | (b3w[0] & ~tmask)) + x[0], e1 = c1 + ((b4w[1] & tmask) | (b3w[1] & ~tmask)) + x[1];
+  const u32 e2 = c2 + ((b4w[2] & tmask) | (b3w[2] & ~tmask)) + x[2], e3 = c3 + ((b4w[3] & tmask) | (b3w[3] & ~tmask)) + x[3];
   out[0] = (e0 & EXP_MASK2) | (__builtin_amdgcn_perm(shi, slo, 0x04040000u) & ~EXP_MASK2);
   out[1] = (e1 & EXP_MASK2) | (__builtin_amdgcn_perm(shi, slo, 0x05050101u) & ~EXP_MASK2);
   out[2] = (e2 & EXP_MASK2) | (__builtin_amdgcn_perm(shi, slo, 0x06060202u) & ~EXP_MASK2);
@@ -183,7 +194,7 @@ __device__ __forceinline__ void decode_unit_x(u32 slo, u32 shi, u32 g24, bool t0
 }
 // raw group: 8 x 5 high exponent bits (40-bit little endian in lo/hi) as exponent-field words MINUS the 4-bit base words,
 // so that code + base4 + x reproduces code | hi5 << 3 exactly (32-bit arithmetic, the base cancels)
-__device__ __forceinline__ u32x4 raw_x_words(u32 lo, u32 hi, const u32* __restrict__ b4w) {
+__device__ __forceinline__ u32x4 raw_x_words(u32 lo, u32 hi, const u32x4& b4w) {
   u32x4 x;
   x[0] = (((lo) & 31u) << 10 | ((lo >> 20) & 31u) << 26) - b4w[0];
   x[1] = (((lo >> 5) & 31u) << 10 | ((lo >> 25) & 31u) << 26) - b4w[1];
@@ -192,74 +203,73 @@ __device__ __forceinline__ u32x4 raw_x_words(u32 lo, u32 hi, const u32* __restri
   return x;
 }
 
-__device__ __forceinline__ void consume_tile(const TileRegs& R, WaveState& st, AttnLds& L, const Bases& B,
-                                             u32 kto, u32 vto, int tile, int S, float scale_log2e, int a, int q,
-                                             const u32x4 (&qf)[4], const u32 (&kb3)[4][4], const u32 (&kb4)[4][4],
-                                             const u32 (&vb3)[4], const u32 (&vb4)[4]) {
-  // ---- K escapes: spread the lane's 4-bit-group bytes to units, expand through the table
-  const u32 ktag8 = __builtin_amdgcn_ubfe(R.kf, 8 * q, 8);
-  u32x4 x[4];
-  {
-    const u32 eb4 = __builtin_amdgcn_perm(0u, R.ke[0], L.sel[ktag8 & 0x55u]);
+// The x words of the lane's four units.  Common case: 4-bit groups only -> one v_perm + four table reads.  A wave with a raw
+// group somewhere (most tiles, few lanes) patches those units from the prefetched bytes; a lane with two or more raw groups
+// (its bytes may not fit the 8 prefetched ones) re-reads memory.
+template <int KIND>
+__device__ __forceinline__ void unit_x_words(const KindRegs& R, const AttnLds& L, const uint8_t* __restrict__ esc_tile, int q,
+                                             const u32x4* __restrict__ b4w /* K: [4] per unit, V: [1] */, u32& tag8, u32x4* __restrict__ x) {
+  tag8 = __builtin_amdgcn_ubfe(R.f, 8 * q, 8);
+  const u32 eb4 = __builtin_amdgcn_perm(R.e[1], R.e[0], L.sel[tag8]);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) x[u] = L.xlut[(eb4 >> (8 * u)) & 0xFFu];
-  }
-  if (__builtin_amdgcn_ballot_w64((ktag8 & 0xAAu) != 0u)) {      // some lane holds a raw group (rare per lane, common per tile)
-    if (ktag8 & 0xAAu) {                                          // redo every escaped unit of this lane at its true offset
+  for (int u = 0; u < 4; ++u) x[u] = L.xlut[(eb4 >> (8 * u)) & 0xFFu];
+  if (__builtin_amdgcn_ballot_w64((tag8 & 0xAAu) != 0u)) {
+    const u64 e64 = (u64)R.e[0] | ((u64)R.e[1] << 32);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (((tag8 >> (2 * u)) & 3u) == 3u) {          // offset = number of 4-bit groups below (a raw one below is handled next)
+        const u64 v = e64 >> (8 * __popc(tag8 & (0x55u & ((1u << (2 * u)) - 1u))));
+        x[u] = raw_x_words((u32)v, (u32)(v >> 32), b4w[KIND == KIND_K ? u : 0]);
+      }
+    }
+    if (__popc(tag8 & 0xAAu) >= 2) {
       u32 off = 0u;
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        const u32 t = (ktag8 >> (2 * u)) & 3u;
+        const u32 t = (tag8 >> (2 * u)) & 3u;
         if (t) {
-          u32 lo, hi;
-          if (off + (u32)tag_size(t) <= 8u) {
-            const u64 v = ((u64)R.ke[0] | ((u64)R.ke[1] << 32)) >> (8u * off);
-            lo = (u32)v; hi = (u32)(v >> 32);
-          } else {
-            const u64 v = load_u64_unaligned(B.kov + kto + R.kpos0 + off);
-            lo = (u32)v; hi = (u32)(v >> 32);
-          }
-          x[u] = t == 1u ? L.xlut[lo & 0xFFu] : raw_x_words(lo, hi, kb4[u]);
+          const u64 v = load_u64_unaligned(esc_tile + R.pos0 + off);
+          x[u] = t == 1u ? L.xlut[(u32)v & 0xFFu] : raw_x_words((u32)v, (u32)(v >> 32), b4w[KIND == KIND_K ? u : 0]);
         }
         off += (u32)tag_size(t);
       }
     }
   }
+}
+
+__device__ __forceinline__ u32 tier_mask(u32 tag8, int u) { return (u32)__builtin_amdgcn_sbfe((int)tag8, 2 * u, 1); }   // 0 or ~0
+
+// PARTIAL: the tile is the last one of the sequence and only partly filled (rows >= S are masked out).  It is a template
+// parameter, not a run-time branch, so that no branch separates the score MFMAs from the first read of their result.
+template <bool PARTIAL>
+__device__ __forceinline__ void consume_tile(const TileRegs& R, WaveState& st, const AttnLds& L, const Bases& B,
+                                             u32 kto, u32 vto, int tile, int S, float scale_log2e, int a, int q,
+                                             const u32x4 (&qf)[4], const u32x4 (&kb3)[4], const u32x4 (&kb4)[4],
+                                             const u32x4& vb3, const u32x4& vb4) {
+  u32 ktag8, vtag8;
+  u32x4 xk[4], xv[4];
+  unit_x_words<KIND_K>(R.k, L, B.kov + kto, q, kb4, ktag8, xk);
+  unit_x_words<KIND_V>(R.v, L, B.vov + vto, q, &vb4, vtag8, xv);
   // ---- scores: S[tok 4q+r][head a]
   f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
     u32 slo, shi, w[4];
-    unit_sm(R.k, u, slo, shi);
-    decode_unit_x(slo, shi, unit_code_word(R.k.c0, R.k.c1, R.k.c2, u), ((ktag8 >> (2 * u)) & 1u) == 0u, x[u], kb3[u], kb4[u], w);
+    unit_sm(R.k.pay, u, slo, shi);
+    decode_unit_x(slo, shi, unit_code_word(R.k.pay.c0, R.k.pay.c1, R.k.pay.c2, u), tier_mask(ktag8, u), xk[u], kb3[u], kb4[u], w);
     const u32x4 av = {w[0], w[1], w[2], w[3]};
     sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av), __builtin_bit_cast(bf16x8, qf[u]), sacc, 0, 0, 0);
   }
-  // ---- V escapes (each unit has its own 8 bytes)
-#pragma unroll
-  for (int u = 0; u < 4; ++u) {
-    const bool t0 = ((R.vt8 >> (2 * u)) & 1u) == 0u;
-    x[u] = L.xlut[t0 ? 0u : (R.ve[u][0] & 0xFFu)];
-  }
-  if (__builtin_amdgcn_ballot_w64((R.vt8 & 0xAAu) != 0u)) {
-#pragma unroll
-    for (int u = 0; u < 4; ++u)
-      if (((R.vt8 >> (2 * u)) & 3u) == 3u) x[u] = raw_x_words(R.ve[u][0], R.ve[u][1], vb4);
-  }
-  // ---- online softmax per head a over the tile's 16 tokens (4 in this lane, 4 quads), base 2
+  // ---- online softmax per head a over the tile's 16 tokens (4 in this lane, 4 quads); exp2(score * scale*log2e - mu)
   const int tok0 = tile * T + 4 * q;
-  float s[4];
+  if (PARTIAL) {
 #pragma unroll
-  for (int r = 0; r < 4; ++r) s[r] = sacc[r] * scale_log2e;
-  const bool partial = tile * T + T > S;          // uniform: only the last tile of a sequence can be partly filled
-  if (partial) {
-#pragma unroll
-    for (int r = 0; r < 4; ++r) if (tok0 + r >= S) s[r] = -INFINITY;
+    for (int r = 0; r < 4; ++r) sacc[r] = tok0 + r >= S ? -INFINITY : sacc[r];
   }
-  const float tmax = quad_rows_max(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])));
+  const float tmax = quad_rows_max(fmaxf(fmaxf(sacc[0], sacc[1]), fmaxf(sacc[2], sacc[3])));
   if (__builtin_amdgcn_ballot_w64(tmax > st.m_run)) {             // the running maximum of some head grows (rare after the first tiles)
-    const float mn = fmaxf(st.m_run, tmax), mu = mn == -INFINITY ? 0.f : mn;
-    const float alpha = __builtin_amdgcn_exp2f(st.m_run - mu);
+    const float mn = fmaxf(st.m_run, tmax), mu = mn == -INFINITY ? 0.f : mn * scale_log2e;
+    const float alpha = __builtin_amdgcn_exp2f(st.m_run == -INFINITY ? -INFINITY : st.mu_run - mu);
     st.l_run *= alpha;
 #pragma unroll
     for (int i = 0; i < 8; ++i) st.acc[i] *= alpha;
@@ -267,7 +277,7 @@ __device__ __forceinline__ void consume_tile(const TileRegs& R, WaveState& st, A
   }
   float p[4];
 #pragma unroll
-  for (int r = 0; r < 4; ++r) p[r] = __builtin_amdgcn_exp2f(s[r] - st.mu_run);
+  for (int r = 0; r < 4; ++r) p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[r], scale_log2e, -st.mu_run));
   st.l_run += (p[0] + p[1]) + (p[2] + p[3]);
   const u32x2 pw = {pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3])};
   const s16x4 pb = __builtin_bit_cast(s16x4, pw);
@@ -276,13 +286,14 @@ __device__ __forceinline__ void consume_tile(const TileRegs& R, WaveState& st, A
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
     u32 slo, shi;
-    unit_sm(R.v, u, slo, shi);
-    decode_unit_x(slo, shi, unit_code_word(R.v.c0, R.v.c1, R.v.c2, u), ((R.vt8 >> (2 * u)) & 1u) == 0u, x[u], vb3, vb4, W[u]);
+    unit_sm(R.v.pay, u, slo, shi);
+    decode_unit_x(slo, shi, unit_code_word(R.v.pay.c0, R.v.pay.c1, R.v.pay.c2, u), tier_mask(vtag8, u), xv[u], vb3, vb4, W[u]);
   }
-  if (partial) {                // rows beyond the sequence must not reach the product
+  if (PARTIAL) {                // rows beyond the sequence must not reach the product
 #pragma unroll
     for (int u = 0; u < 4; ++u)
-      if (tok0 + u >= S) { W[u][0] = W[u][1] = W[u][2] = W[u][3] = 0u; }
+#pragma unroll
+      for (int pp = 0; pp < 4; ++pp) W[u][pp] = tok0 + u >= S ? 0u : W[u][pp];
   }
 #pragma unroll
   for (int pp = 0; pp < 4; ++pp) {
@@ -300,91 +311,83 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
   const int b = bh / A.n_kv, kvh = bh % A.n_kv, G = A.G;
   const int slot = A.slot[b], ch = (slot < 0 ? 0 : slot) * A.n_kv + kvh;
   if (split == A.nsplit) { tail_block(A, b, kvh, ch, slot); return; }
-  build_luts(L, tid);
+  const long qh0 = (long)b * A.n_q + (long)kvh * G;
+  build_tables(L, tid, A, ch % A.NB, qh0);
 
   const int S = slot < 0 ? 0 : A.sl[ch];
   const int ntiles = (S + T - 1) / T, chunk = (ntiles + A.nsplit - 1) / A.nsplit;
   const int tlo = split * chunk, thi = min(tlo + chunk, ntiles);
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, a = lane & 15, q = lane >> 4;
   const long rowb = (long)ch * A.S_pad, tileb = (long)ch * (A.S_pad / T);
-  const long qh0 = (long)b * A.n_q + (long)kvh * G;
   Bases B;
   B.ksm = A.k.sm + rowb * D; B.kcd = A.k.cd + rowb * CB; B.kfl = A.k.flags + rowb; B.kto = A.k.tile_off + tileb; B.kov = A.k.ovf + A.k.head_start[ch];
   B.vsm = A.v.sm + rowb * D; B.vcd = A.v.cd + rowb * CB; B.vfl = A.v.flags + rowb; B.vto = A.v.tile_off + tileb; B.vov = A.v.ovf + A.v.head_start[ch];
 
-  // Q as the B operand of the score product: lane (head a, quad q), product u covers group 4q+u in word order (e, e+4)
-  u32x4 qf[4];
-#pragma unroll
-  for (int u = 0; u < 4; ++u) {
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-      u32 w = 0u;
-      if (a < G) {
-        const u16* qp = A.q + (qh0 + a) * D;
-        w = (u32)qp[chan_k(8 * (4 * q + u) + p)] | ((u32)qp[chan_k(8 * (4 * q + u) + p + 4)] << 16);
-      }
-      qf[u][p] = w;
-    }
+  // tiles of this wave: t(i) = tlo + wave + 4 i, i < n.  Ping-pong registers R0/R1; tag words are fetched one tile further
+  // ahead (index clamped to the wave's last tile, so that no load sits under a branch the consumer has to join).  A partly
+  // filled last tile of the sequence is taken out of the pipeline and handled at the end by the wave that owns it.
+  const int t0 = tlo + wave;
+  const int n_all = t0 < thi ? (thi - t0 + 3) / 4 : 0;
+  const bool own_partial = n_all > 0 && (S % T) != 0 && t0 + 4 * (n_all - 1) == ntiles - 1;
+  const int n = n_all - (own_partial ? 1 : 0);
+  const int tlast = t0 + 4 * (n - 1);
+  TileRegs R0, R1;
+  TagRegs Tg, TgC0, TgC1;
+  if (n > 0) {          // start the first tile's loads before waiting for the block tables
+    load_tags(B, t0, a, Tg);
+    TgC0 = Tg;
+    load_tile(B, t0, lane, Tg, R0);
+    load_tags(B, min(t0 + 4, tlast), a, Tg);
   }
+  __syncthreads();        // block tables are ready
+  // Q as the B operand of the score product: lane (head a, quad q), product u covers group 4q+u in word order (e, e+4);
   // exponent-base words of the lane's units
-  const int brow = ch % A.NB;
-  u32 kb3[4][4], kb4[4][4], vb3[4], vb4[4];
+  u32x4 qf[4], kb3[4], kb4[4];
 #pragma unroll
-  for (int u = 0; u < 4; ++u) {
-    load_base_words<KIND_K>(A.k.base3 + (long)brow * D, 4 * q + u, kb3[u]);
-    load_base_words<KIND_K>(A.k.base4 + (long)brow * D, 4 * q + u, kb4[u]);
-  }
-  load_base_words<KIND_V>(A.v.base3 + (long)brow * D, a, vb3);
-  load_base_words<KIND_V>(A.v.base4 + (long)brow * D, a, vb4);
-  u32 bperm_addr[4];
-#pragma unroll
-  for (int u = 0; u < 4; ++u) bperm_addr[u] = (u32)(4 * (4 * q + u));
-  __syncthreads();        // lookup tables are ready
+  for (int u = 0; u < 4; ++u) { qf[u] = L.qw[a][4 * q + u]; kb3[u] = L.bwk[0][4 * q + u]; kb4[u] = L.bwk[1][4 * q + u]; }
+  const u32x4 vb3 = L.bwv[0][a], vb4 = L.bwv[1][a];
 
   WaveState st;
 #pragma unroll
   for (int i = 0; i < 8; ++i) st.acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   st.m_run = -INFINITY; st.mu_run = 0.f; st.l_run = 0.f;
 
-  // tiles of this wave: t(i) = tlo + wave + 4 i, i < n.  Ping-pong registers R0/R1; tag words are fetched one tile further
-  // ahead (index clamped to the wave's last tile, so that no load sits under a branch the consumer has to join).
-  const int t0 = tlo + wave;
-  const int n = t0 < thi ? (thi - t0 + 3) / 4 : 0;
   if (n > 0) {
-    const int tlast = t0 + 4 * (n - 1);
-    TileRegs R0, R1;
-    TagRegs Tg, TgC0, TgC1;
-    load_tags(B, t0, S, a, Tg);
-    TgC0 = Tg;
-    load_tile(B, t0, lane, Tg, bperm_addr, R0);
-    load_tags(B, min(t0 + 4, tlast), S, a, Tg);
     int i = 0;
     for (; i + 2 < n; i += 2) {
       const int t = t0 + 4 * i;
       TgC1 = Tg;
-      load_tile(B, t + 4, lane, Tg, bperm_addr, R1);
-      load_tags(B, min(t + 8, tlast), S, a, Tg);
-      consume_tile(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+      load_tile(B, t + 4, lane, Tg, R1);
+      load_tags(B, min(t + 8, tlast), a, Tg);
+      consume_tile<false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
       TgC0 = Tg;
-      load_tile(B, t + 8, lane, Tg, bperm_addr, R0);
-      load_tags(B, min(t + 12, tlast), S, a, Tg);
-      consume_tile(R1, st, L, B, TgC1.kto, TgC1.vto, t + 4, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+      load_tile(B, t + 8, lane, Tg, R0);
+      load_tags(B, min(t + 12, tlast), a, Tg);
+      consume_tile<false>(R1, st, L, B, TgC1.kto, TgC1.vto, t + 4, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
     }
     const int t = t0 + 4 * i;
     if (n - i == 2) {
       TgC1 = Tg;
-      load_tile(B, t + 4, lane, Tg, bperm_addr, R1);
-      consume_tile(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
-      consume_tile(R1, st, L, B, TgC1.kto, TgC1.vto, t + 4, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+      load_tile(B, t + 4, lane, Tg, R1);
+      consume_tile<false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+      consume_tile<false>(R1, st, L, B, TgC1.kto, TgC1.vto, t + 4, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
     } else {
-      consume_tile(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+      consume_tile<false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
     }
   }
-  float m_run = st.m_run, l_run = st.l_run;
+  if (own_partial) {
+    const int t = ntiles - 1;
+    load_tags(B, t, a, Tg);
+    load_tile(B, t, lane, Tg, R0);
+    consume_tile<true>(R0, st, L, B, Tg.kto, Tg.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+  }
+  // The accumulators are MFMA results: keep their first non-MFMA read a full MFMA latency away on every path.
+  asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");
+  float l_run = quad_rows_sum(st.l_run);
+  const float m_run = st.m_run == -INFINITY ? -INFINITY : st.mu_run;     // partial maxima are stored in the base-2 domain
   f32x4 (&acc)[8] = st.acc;
 
   // ---- merge the 4 waves of the block, write the split's partial
-  l_run = quad_rows_sum(l_run);
   if (a < G) {
     if (q == 0) { L.m[wave][a] = m_run; L.l[wave][a] = l_run; }
 #pragma unroll
@@ -411,34 +414,46 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
 }
 
 // ---------------------------------------------------------------------------------------------------- split merge
-__global__ void __launch_bounds__(128) k_attn_combine(const float* __restrict__ pm, const float* __restrict__ pl, const float* __restrict__ pa,
+__global__ void __launch_bounds__(512) k_attn_combine(const float* __restrict__ pm, const float* __restrict__ pl, const float* __restrict__ pa,
                                                       u16* __restrict__ out, int nslot) {
   __shared__ float fs[MAX_SLOTS];
-  __shared__ float red[2];
-  const int qh = blockIdx.x, tid = threadIdx.x;
+  __shared__ float red[8];
+  __shared__ float part[3][D];
+  const int qh = blockIdx.x, tid = threadIdx.x, wv = tid >> 6;
   float m = -INFINITY;
-  for (int s = tid; s < nslot; s += 128) m = fmaxf(m, pm[(long)qh * nslot + s]);
+  for (int s = tid; s < nslot; s += 512) m = fmaxf(m, pm[(long)qh * nslot + s]);
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
-  if ((tid & 63) == 0) red[tid >> 6] = m;
+  if ((tid & 63) == 0) red[wv] = m;
   __syncthreads();
-  const float M = fmaxf(red[0], red[1]);
+  float M = red[0];
+#pragma unroll
+  for (int w = 1; w < 8; ++w) M = fmaxf(M, red[w]);
   __syncthreads();
   float l = 0.f;
-  for (int s = tid; s < nslot; s += 128) {
+  for (int s = tid; s < nslot; s += 512) {
     const float v = pm[(long)qh * nslot + s];
     const float f = v == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(v - M);
     fs[s] = f; l += pl[(long)qh * nslot + s] * f;
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o, 64);
-  if ((tid & 63) == 0) red[tid >> 6] = l;
+  if ((tid & 63) == 0) red[wv] = l;
   __syncthreads();
-  const float L = red[0] + red[1];
+  float Lsum = 0.f;
+#pragma unroll
+  for (int w = 0; w < 8; ++w) Lsum += red[w];
+  const int d = tid & 127, part_id = tid >> 7;      // four slot-interleaved partial sums per output element
   float acc = 0.f;
-  for (int s = 0; s < nslot; ++s) acc += pa[((long)qh * nslot + s) * D + tid] * fs[s];
-  const float o = L > 0.f ? acc / L : 0.f;
-  out[(long)qh * D + tid] = __builtin_bit_cast(u16, (__bf16)o);
+#pragma unroll 4
+  for (int s = part_id; s < nslot; s += 4) acc += pa[((long)qh * nslot + s) * D + d] * fs[s];
+  if (part_id) part[part_id - 1][d] = acc;
+  __syncthreads();
+  if (part_id == 0) {
+    acc += part[0][d] + part[1][d] + part[2][d];
+    const float o = Lsum > 0.f ? acc / Lsum : 0.f;
+    out[(long)qh * D + d] = __builtin_bit_cast(u16, (__bf16)o);
+  }
 }
 
 }  // namespace gaac
@@ -480,7 +495,7 @@ extern "C" int gaac_attn_split(
 
 extern "C" int gaac_attn_combine(const float* pm, const float* pl, const float* pa, void* out, int n_rows, int nslot, void* stream) {
   GAAC_REQUIRE(pm && pl && pa && out && n_rows > 0 && nslot >= 1 && nslot <= MAX_SLOTS, "gaac_attn_combine: bad arguments");
-  hipLaunchKernelGGL(k_attn_combine, dim3(n_rows), dim3(128), 0, (hipStream_t)stream, pm, pl, pa, (u16*)out, nslot);
+  hipLaunchKernelGGL(k_attn_combine, dim3(n_rows), dim3(512), 0, (hipStream_t)stream, pm, pl, pa, (u16*)out, nslot);
   return launch_status("gaac_attn(combine)");
 }
 

@@ -116,9 +116,9 @@ __global__ void __launch_bounds__(64) k_decode_tiles(const uint8_t* __restrict__
   const long row0 = (long)h * S_pad + (long)tile * T;
   Payload P;
   load_payload(sm + row0 * D, cd + row0 * CB, lane, P);
-  const u32 tag_word = (tile * T + a < S) ? (u32)flags[row0 + a] : 0u;
+  const u32 tag_word = (u32)flags[row0 + a];      // rows beyond S carry tag 0 (the encoder writes every word of a tile)
   UnitMeta M;
-  tile_unit_meta<KIND>(tag_word, lane, M);
+  tile_unit_meta(tag_word, lane, M);
   const uint8_t* esc = ovf + head_start[h] + tile_off[(long)h * (S_pad / T) + tile];
   u32 b3w[4], b4w[4];
   if (KIND == KIND_V) { load_base_words<KIND>(base3 + (long)brow * D, a, b3w); load_base_words<KIND>(base4 + (long)brow * D, a, b4w); }

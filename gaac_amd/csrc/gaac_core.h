@@ -12,8 +12,11 @@
 // Native byte order of a tile:
 //   sign/mantissa (2048 B): byte 1024*j + 16*l + 8*v + i  = element i of unit 2j+v of lane l   (j,v in {0,1})
 //   codes (768 B):          byte 256*k + 4*l + b          = byte 4k+b of the lane's 12 code bytes (unit u -> bytes 3u..3u+2)
-// Tag words stay token-major (one u32 per token row, 2 bits per group) and the escape stream keeps the reference
-// order (rows ascending, groups ascending; 1 byte per 4-bit group, 5 bytes per raw group).
+// Tag words (16 x u32 per tile) and escape bytes are stored per LINE a = l & 15 of the tile: word a holds the 2-bit tags
+// of the 16 units of line a, unit (a, j) at bits 2j (lane a+16q owns bits 8q..8q+7); the tile's escape bytes follow line
+// order (a ascending, j ascending; 1 byte per 4-bit group, 5 bytes per raw group).  For K a line is a token row and j the
+// group, which IS the reference order; for V a line is a group and j the token, i.e. the 16 x 16 tag matrix and the
+// escape order of a V tile are the transpose of the reference's.  Tile offsets and per-tile byte counts are unaffected.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>

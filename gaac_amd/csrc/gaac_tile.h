@@ -31,7 +31,7 @@ __device__ __forceinline__ void stage_bases(EncodeLds& L, const uint8_t* __restr
   if (lane < T) L.tags[lane] = 0u;
 }
 
-// Encodes the tile staged in L (after a barrier).  Writes the native sign/mantissa and code bytes, the 16 tag words and
+// Encodes the tile staged in L (after a barrier).  Writes the native sign/mantissa and code bytes, the 16 tag words (one per line) and
 // the escape bytes (at esc_dst + offset-in-tile; nullptr = count only).  Returns the tile's escape byte count (all lanes).
 // Must be called by all 64 lanes of a one-wave block: it uses block barriers.
 template <int KIND>
@@ -66,8 +66,9 @@ __device__ __forceinline__ int encode_staged_tile(EncodeLds& L, int nvalid, int 
     g24[u] = !valid ? 0u : (fit3 ? c3 : (fit4 ? c4 : cr));
     slo[u] = valid ? s_lo : 0u; shi[u] = valid ? s_hi : 0u;
     eb[u] = e4; hi40[u] = h;
-    if (tag[u]) atomicOr(&L.tags[tok], tag[u] << (2 * grp));
   }
+  // tag word of line a: this lane owns bits 8q..8q+7 (its four units)
+  reinterpret_cast<uint8_t*>(L.tags)[4 * a + q] = (uint8_t)(tag[0] | (tag[1] << 2) | (tag[2] << 4) | (tag[3] << 6));
   u32x4 s0 = {slo[0], shi[0], slo[1], shi[1]}, s1 = {slo[2], shi[2], slo[3], shi[3]};
   *reinterpret_cast<u32x4*>(sm_tile + 16 * lane) = s0;
   *reinterpret_cast<u32x4*>(sm_tile + 1024 + 16 * lane) = s1;
@@ -82,16 +83,14 @@ __device__ __forceinline__ int encode_staged_tile(EncodeLds& L, int nvalid, int 
   }
   __syncthreads();
   if (esc_dst) {
+    uint8_t* p = esc_dst + L.rowoff[a] + esc_prefix(L.tags[a], 8 * q);
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
-      if (tag[u]) {
-        const int tok = unit_token<KIND>(a, q, u), grp = unit_group<KIND>(a, q, u);
-        uint8_t* p = esc_dst + L.rowoff[tok] + esc_prefix(L.tags[tok], 2 * grp);
-        if (tag[u] == 1u) p[0] = (uint8_t)eb[u];
-        else {
+      if (tag[u] == 1u) { p[0] = (uint8_t)eb[u]; p += 1; }
+      else if (tag[u] == 3u) {
 #pragma unroll
-          for (int k = 0; k < 5; ++k) p[k] = (uint8_t)(hi40[u] >> (8 * k));
-        }
+        for (int k = 0; k < 5; ++k) p[k] = (uint8_t)(hi40[u] >> (8 * k));
+        p += 5;
       }
     }
   }
@@ -99,26 +98,14 @@ __device__ __forceinline__ int encode_staged_tile(EncodeLds& L, int nvalid, int 
 }
 
 // Per-lane metadata of a stored tile: the 2-bit tag of each of the lane's four units and the offset of the unit's escape
-// bytes from the start of the tile's escape bytes.  tag_word = this lane's token-major tag word flags_tile[lane & 15]
-// (already zeroed for rows beyond the sequence).
+// bytes from the start of the tile's escape bytes.  tag_word = the tag word of the lane's line, flags_tile[lane & 15].
 struct UnitMeta { u32 tag[4]; int pos[4]; };
-template <int KIND>
 __device__ __forceinline__ void tile_unit_meta(u32 tag_word, int lane, UnitMeta& M) {
-  const int a = lane & 15, q = lane >> 4;
+  const int q = lane >> 4;
   const u32 rb = (u32)esc_bytes(tag_word);
-  const int rowoff = (int)(row_scan16(rb) - rb);
-  if (KIND == KIND_K) {
-    int pos = rowoff + esc_prefix(tag_word, 8 * q);
+  int pos = (int)(row_scan16(rb) - rb) + esc_prefix(tag_word, 8 * q);
 #pragma unroll
-    for (int u = 0; u < 4; ++u) { M.tag[u] = (tag_word >> (8 * q + 2 * u)) & 3u; M.pos[u] = pos; pos += tag_size(M.tag[u]); }
-  } else {
-#pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const u32 f = (u32)__shfl((int)tag_word, 4 * q + u, 64);
-      const int ro = __shfl(rowoff, 4 * q + u, 64);
-      M.tag[u] = (f >> (2 * a)) & 3u; M.pos[u] = ro + esc_prefix(f, 2 * a);
-    }
-  }
+  for (int u = 0; u < 4; ++u) { M.tag[u] = (tag_word >> (8 * q + 2 * u)) & 3u; M.pos[u] = pos; pos += tag_size(M.tag[u]); }
 }
 
 }  // namespace gaac
