@@ -29,6 +29,7 @@ struct AttnArgs {
   const int* slot; const int* sl;
   int S_pad; float scale_log2e; int nsplit; int nslot; int n_kv; int n_q; int G; int NB;
   const u16* kt; const u16* vt; const int* tl; int tcap;
+  int* tickets; u16* out;      // fused merge: one arrival counter per (batch row, kv head), zero between launches
 };
 
 __device__ __forceinline__ float bf16_bits_to_float(u32 h) { return __uint_as_float(h << 16); }
@@ -36,6 +37,72 @@ __device__ __forceinline__ u32 pack_bf16x2(float lo, float hi) {
   typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
   bf16x2 v; v[0] = (__bf16)lo; v[1] = (__bf16)hi;
   return __builtin_bit_cast(u32, v);
+}
+
+// ---------------------------------------------------------------------------------------------------- fused merge
+// Merge of the split partials (gaac_combine, /root/reference/gaac/kernel.py:281-294) by the LAST block of a (batch row, kv head)
+// to finish: every block publishes its partial, then takes a ticket; the block that draws the last ticket merges all NSLOT
+// partials of the G query heads and re-arms the counter.  One wave per head, no block-wide synchronisation inside.
+// The partials travel between blocks on different XCDs (one L2 each) inside one kernel, so they are written and read with
+// agent-scope accesses (write-through stores, cache-bypassing loads) instead of whole-L2 write-back/invalidate fences.
+typedef __attribute__((ext_vector_type(4))) float f32x4v;
+__device__ __forceinline__ void store_partial(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ float load_partial(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+constexpr int AUX_AGENT_SCOPE = 0x10;      // sc1 of the gfx94x/gfx950 buffer cache policy
+__device__ __forceinline__ void merge_head_by_wave(const AttnArgs& A, long row, float* __restrict__ fs, int lane) {
+  const int nslot = A.nslot;
+  const float* pm = A.pm + row * nslot; const float* pl = A.pl + row * nslot;
+  const float* pa = A.pa + row * nslot * D;
+  float m = -INFINITY;
+  for (int s = lane; s < nslot; s += 64) m = fmaxf(m, load_partial(pm + s));
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  float l = 0.f;
+  for (int s = lane; s < nslot; s += 64) {
+    const float v = load_partial(pm + s);
+    const float f = v == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(v - m);
+    fs[s] = f; l += load_partial(pl + s) * f;
+  }
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o, 64);
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  const int sg = lane >> 5, dq = (lane & 31) * 4;      // two slots per wave-wide load, four dims per lane
+  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(pa), 0, nslot * D * 4, 0x00027000);
+  f32x4v acc = {0.f, 0.f, 0.f, 0.f};
+  constexpr int CH = 16;
+  for (int s0 = sg; s0 < nslot; s0 += 2 * CH) {
+    u32x4 v[CH];
+#pragma unroll
+    for (int k = 0; k < CH; ++k)      // slots past the end are out of the buffer's range and read as zero
+      v[k] = __builtin_amdgcn_raw_buffer_load_b128(rs, ((s0 + 2 * k) * D + dq) * 4, 0, AUX_AGENT_SCOPE);
+#pragma unroll
+    for (int k = 0; k < CH; ++k) {
+      const int s = s0 + 2 * k; const float f = s < nslot ? fs[s] : 0.f;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) acc[c] += __uint_as_float(v[k][c]) * f;
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < 4; ++c) acc[c] += __shfl_xor(acc[c], 32, 64);
+  if (sg == 0) {
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    u32x2 o = {pack_bf16x2(acc[0] * inv, acc[1] * inv), pack_bf16x2(acc[2] * inv, acc[3] * inv)};
+    *reinterpret_cast<u32x2*>(A.out + row * D + dq) = o;
+  }
+}
+// Called by all 256 threads of a block after its partial has been written with store_partial().
+__device__ __forceinline__ void publish_and_merge(const AttnArgs& A, int bh, long qh0, int G, int tid) {
+  __shared__ float fs[4][MAX_SLOTS];
+  __shared__ int last;
+  if (!A.tickets) return;
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // this thread's write-through stores have reached device scope
+  __syncthreads();
+  if (tid == 0) last = atomicAdd(&A.tickets[bh], 1) == A.nslot - 1;
+  __syncthreads();
+  if (!last) return;
+  const int wave = tid >> 6, lane = tid & 63;
+  for (int g = wave; g < G; g += 4) merge_head_by_wave(A, qh0 + g, fs[wave], lane);
+  if (tid == 0) __hip_atomic_store(&A.tickets[bh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);      // re-arm for the next launch
 }
 
 // ---------------------------------------------------------------------------------------------------- raw tail block
@@ -78,7 +145,7 @@ __device__ void tail_block(const AttnArgs& A, int b, int kvh, int ch, int slot) 
     __syncthreads();
     if (g < G) {
       sc[g][tk] = p;
-      if (tk == 0) { const long pidx = (qh0 + g) * A.nslot + (A.nslot - 1); A.pm[pidx] = m; A.pl[pidx] = l; }
+      if (tk == 0) { const long pidx = (qh0 + g) * A.nslot + (A.nslot - 1); store_partial(A.pm + pidx, m); store_partial(A.pl + pidx, l); }
     }
   }
   __syncthreads();
@@ -86,8 +153,9 @@ __device__ void tail_block(const AttnArgs& A, int b, int kvh, int ch, int slot) 
   for (int g = tid >> 7; g < G; g += 2) {
     float acc = 0.f;
     for (int tk = 0; tk < TL; ++tk) acc += sc[g][tk] * bf16_bits_to_float(A.vt[base + (long)tk * D + d]);
-    A.pa[((qh0 + g) * A.nslot + (A.nslot - 1)) * D + d] = acc;
+    store_partial(A.pa + ((qh0 + g) * A.nslot + (A.nslot - 1)) * D + d, acc);
   }
+  publish_and_merge(A, b * A.n_kv + kvh, qh0, G, tid);
 }
 
 // ---------------------------------------------------------------------------------------------------- block tables (LDS)
@@ -104,7 +172,27 @@ struct AttnLds {
   float m[4][GMAX], l[4][GMAX];
   float acc[4][GMAX][D];
 };
-__device__ __forceinline__ void build_tables(AttnLds& L, int tid, const AttnArgs& A, int brow, long qh0) {
+struct TableRegs { u32 b0, b1; u32 qlo[4], qhi[4]; };      // one thread's raw inputs of the per-block tables
+// global loads only (issued before the first tile's loads so that the two latencies overlap)
+__device__ __forceinline__ void tables_load(TableRegs& Tr, int tid, const AttnArgs& A, int brow, long qh0) {
+  {   // one base word per thread: kind = tid >> 7, tier = (tid >> 6) & 1, group = (tid >> 2) & 15, p = tid & 3
+    const int kind = tid >> 7, tier = (tid >> 6) & 1, g = (tid >> 2) & 15, p = tid & 3;
+    const StoreView& st = kind ? A.v : A.k;
+    const uint8_t* row = (tier ? st.base4 : st.base3) + (long)brow * D;
+    const int c0 = kind ? chan_v(8 * g + p) : chan_k(8 * g + p), c1 = kind ? chan_v(8 * g + p + 4) : chan_k(8 * g + p + 4);
+    Tr.b0 = row[c0]; Tr.b1 = row[c1];
+  }
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {      // query words: head = idx >> 6, group = (idx >> 2) & 15, p = idx & 3
+    const int idx = tid + 256 * k, h = idx >> 6, g = (idx >> 2) & 15, p = idx & 3;
+    Tr.qlo[k] = 0u; Tr.qhi[k] = 0u;
+    if (h < A.G) {
+      const u16* qp = A.q + (qh0 + h) * D;
+      Tr.qlo[k] = qp[chan_k(8 * g + p)]; Tr.qhi[k] = qp[chan_k(8 * g + p + 4)];
+    }
+  }
+}
+__device__ __forceinline__ void tables_store(AttnLds& L, const TableRegs& Tr, int tid) {
   {
     const u32 e = (u32)tid;
     u32x4 w;
@@ -120,24 +208,15 @@ __device__ __forceinline__ void build_tables(AttnLds& L, int tid, const AttnArgs
     }
     L.sel[tid] = selw;
   }
-  {   // one base word per thread: kind = tid >> 7, tier = (tid >> 6) & 1, group = (tid >> 2) & 15, p = tid & 3
+  {
     const int kind = tid >> 7, tier = (tid >> 6) & 1, g = (tid >> 2) & 15, p = tid & 3;
-    const StoreView& st = kind ? A.v : A.k;
-    const uint8_t* row = (tier ? st.base4 : st.base3) + (long)brow * D;
-    const int c0 = kind ? chan_v(8 * g + p) : chan_k(8 * g + p), c1 = kind ? chan_v(8 * g + p + 4) : chan_k(8 * g + p + 4);
-    const u32 w = ((u32)row[c0] << 7) | ((u32)row[c1] << 23);
     u32* dst = kind ? reinterpret_cast<u32*>(&L.bwv[tier][g]) : reinterpret_cast<u32*>(&L.bwk[tier][g]);
-    dst[p] = w;
+    dst[p] = (Tr.b0 << 7) | (Tr.b1 << 23);
   }
 #pragma unroll
-  for (int k = 0; k < (GMAX * NG * 4) / 256; ++k) {      // query words: head = idx >> 6, group = (idx >> 2) & 15, p = idx & 3
+  for (int k = 0; k < 4; ++k) {
     const int idx = tid + 256 * k, h = idx >> 6, g = (idx >> 2) & 15, p = idx & 3;
-    u32 w = 0u;
-    if (h < A.G) {
-      const u16* qp = A.q + (qh0 + h) * D;
-      w = (u32)qp[chan_k(8 * g + p)] | ((u32)qp[chan_k(8 * g + p + 4)] << 16);
-    }
-    reinterpret_cast<u32*>(&L.qw[h][g])[p] = w;
+    reinterpret_cast<u32*>(&L.qw[h][g])[p] = Tr.qlo[k] | (Tr.qhi[k] << 16);
   }
 }
 
@@ -180,13 +259,13 @@ __device__ __forceinline__ void load_tile(const Bases& B, int tile, int lane, co
 struct WaveState { f32x4 acc[8]; float m_run, mu_run, l_run; };     // acc[i][r] = O[head a][group 4q+r, element i]; m in raw score units
 
 // unit decode with the escape contribution already expanded to exponent-field words x (see AttnLds::xlut)
-__device__ __forceinline__ void decode_unit_x(u32 slo, u32 shi, u32 g24, u32 tmask, const u32x4& x, const u32x4& b3w, const u32x4& b4w,
+__device__ __forceinline__ void decode_unit_x(u32 slo, u32 shi, u32 g24, bool t0, const u32x4& x, const u32x4& b3w, const u32x4& b4w,
                                               u32* __restrict__ out) {
   const u32 cw = (g24 & 0xFFFu) | ((g24 << 4) & 0x0FFF0000u);
   const u32 c0 = (cw << 7) & 0x03800380u, c1 = (cw << 4) & 0x03800380u, c2 = (cw << 1) & 0x03800380u, c3 = (cw >> 2) & 0x03800380u;
-  // tmask = 0 for a 3-bit group (base3), ~0 otherwise (base4)
-  const u32 e0 = c0 + ((b4w[0] & tmask) | (b3w[0] & ~tmask)) + x[0], e1 = c1 + ((b4w[1] & tmask) | (b3w[1] & ~tmask)) + x[1];
-  const u32 e2 = c2 + ((b4w[2] & tmask) | (b3w[2] & ~tmask)) + x[2], e3 = c3 + ((b4w[3] & tmask) | (b3w[3] & ~tmask)) + x[3];
+  // t0: 3-bit group (base3); otherwise base4 (raw groups: x already holds hi5 - base4)
+  const u32 e0 = c0 + (t0 ? b3w[0] : b4w[0]) + x[0], e1 = c1 + (t0 ? b3w[1] : b4w[1]) + x[1];
+  const u32 e2 = c2 + (t0 ? b3w[2] : b4w[2]) + x[2], e3 = c3 + (t0 ? b3w[3] : b4w[3]) + x[3];
   out[0] = (e0 & EXP_MASK2) | (__builtin_amdgcn_perm(shi, slo, 0x04040000u) & ~EXP_MASK2);
   out[1] = (e1 & EXP_MASK2) | (__builtin_amdgcn_perm(shi, slo, 0x05050101u) & ~EXP_MASK2);
   out[2] = (e2 & EXP_MASK2) | (__builtin_amdgcn_perm(shi, slo, 0x06060202u) & ~EXP_MASK2);
@@ -204,9 +283,10 @@ __device__ __forceinline__ u32x4 raw_x_words(u32 lo, u32 hi, const u32x4& b4w) {
 }
 
 // The x words of the lane's four units.  Common case: 4-bit groups only -> one v_perm + four table reads.  A wave with a raw
-// group somewhere (most tiles, few lanes) patches those units from the prefetched bytes; a lane with two or more raw groups
-// (its bytes may not fit the 8 prefetched ones) re-reads memory.
-template <int KIND>
+// group somewhere (most tiles, few lanes) patches those units from the prefetched bytes.  A lane with two or more raw groups
+// (its bytes may not fit the 8 prefetched ones) re-reads memory: only the SLOW instantiation contains those loads, so the
+// common instantiation has no memory access between the prefetch and the products.
+template <int KIND, bool SLOW>
 __device__ __forceinline__ void unit_x_words(const KindRegs& R, const AttnLds& L, const uint8_t* __restrict__ esc_tile, int q,
                                              const u32x4* __restrict__ b4w /* K: [4] per unit, V: [1] */, u32& tag8, u32x4* __restrict__ x) {
   tag8 = __builtin_amdgcn_ubfe(R.f, 8 * q, 8);
@@ -222,7 +302,7 @@ __device__ __forceinline__ void unit_x_words(const KindRegs& R, const AttnLds& L
         x[u] = raw_x_words((u32)v, (u32)(v >> 32), b4w[KIND == KIND_K ? u : 0]);
       }
     }
-    if (__popc(tag8 & 0xAAu) >= 2) {
+    if (SLOW && __popc(tag8 & 0xAAu) >= 2) {
       u32 off = 0u;
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
@@ -237,26 +317,26 @@ __device__ __forceinline__ void unit_x_words(const KindRegs& R, const AttnLds& L
   }
 }
 
-__device__ __forceinline__ u32 tier_mask(u32 tag8, int u) { return (u32)__builtin_amdgcn_sbfe((int)tag8, 2 * u, 1); }   // 0 or ~0
+__device__ __forceinline__ bool tier0(u32 tag8, int u) { return (tag8 & (1u << (2 * u))) == 0u; }
 
 // PARTIAL: the tile is the last one of the sequence and only partly filled (rows >= S are masked out).  It is a template
 // parameter, not a run-time branch, so that no branch separates the score MFMAs from the first read of their result.
-template <bool PARTIAL>
+template <bool PARTIAL, bool SLOW>
 __device__ __forceinline__ void consume_tile(const TileRegs& R, WaveState& st, const AttnLds& L, const Bases& B,
                                              u32 kto, u32 vto, int tile, int S, float scale_log2e, int a, int q,
                                              const u32x4 (&qf)[4], const u32x4 (&kb3)[4], const u32x4 (&kb4)[4],
                                              const u32x4& vb3, const u32x4& vb4) {
   u32 ktag8, vtag8;
   u32x4 xk[4], xv[4];
-  unit_x_words<KIND_K>(R.k, L, B.kov + kto, q, kb4, ktag8, xk);
-  unit_x_words<KIND_V>(R.v, L, B.vov + vto, q, &vb4, vtag8, xv);
+  unit_x_words<KIND_K, SLOW>(R.k, L, B.kov + kto, q, kb4, ktag8, xk);
+  unit_x_words<KIND_V, SLOW>(R.v, L, B.vov + vto, q, &vb4, vtag8, xv);
   // ---- scores: S[tok 4q+r][head a]
   f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
     u32 slo, shi, w[4];
     unit_sm(R.k.pay, u, slo, shi);
-    decode_unit_x(slo, shi, unit_code_word(R.k.pay.c0, R.k.pay.c1, R.k.pay.c2, u), tier_mask(ktag8, u), xk[u], kb3[u], kb4[u], w);
+    decode_unit_x(slo, shi, unit_code_word(R.k.pay.c0, R.k.pay.c1, R.k.pay.c2, u), tier0(ktag8, u), xk[u], kb3[u], kb4[u], w);
     const u32x4 av = {w[0], w[1], w[2], w[3]};
     sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av), __builtin_bit_cast(bf16x8, qf[u]), sacc, 0, 0, 0);
   }
@@ -287,7 +367,7 @@ __device__ __forceinline__ void consume_tile(const TileRegs& R, WaveState& st, c
   for (int u = 0; u < 4; ++u) {
     u32 slo, shi;
     unit_sm(R.v.pay, u, slo, shi);
-    decode_unit_x(slo, shi, unit_code_word(R.v.pay.c0, R.v.pay.c1, R.v.pay.c2, u), tier_mask(vtag8, u), xv[u], vb3, vb4, W[u]);
+    decode_unit_x(slo, shi, unit_code_word(R.v.pay.c0, R.v.pay.c1, R.v.pay.c2, u), tier0(vtag8, u), xv[u], vb3, vb4, W[u]);
   }
   if (PARTIAL) {                // rows beyond the sequence must not reach the product
 #pragma unroll
@@ -304,6 +384,18 @@ __device__ __forceinline__ void consume_tile(const TileRegs& R, WaveState& st, c
   }
 }
 
+// A tile needs the SLOW instantiation when some lane holds two or more raw groups (about 1 tile in 100 at 0.3 % raw groups).
+template <bool PARTIAL>
+__device__ __forceinline__ void consume(const TileRegs& R, WaveState& st, const AttnLds& L, const Bases& B, u32 kto, u32 vto, int tile,
+                                        int S, float scale_log2e, int a, int q, const u32x4 (&qf)[4], const u32x4 (&kb3)[4],
+                                        const u32x4 (&kb4)[4], const u32x4& vb3, const u32x4& vb4) {
+  const u32 kr = __builtin_amdgcn_ubfe(R.k.f, 8 * q, 8) & 0xAAu, vr = __builtin_amdgcn_ubfe(R.v.f, 8 * q, 8) & 0xAAu;
+  if (__builtin_expect(__builtin_amdgcn_ballot_w64(((kr & (kr - 1u)) | (vr & (vr - 1u))) != 0u) != 0, 0))
+    consume_tile<PARTIAL, true>(R, st, L, B, kto, vto, tile, S, scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+  else
+    consume_tile<PARTIAL, false>(R, st, L, B, kto, vto, tile, S, scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+}
+
 // ---------------------------------------------------------------------------------------------------- main kernel
 __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
   __shared__ AttnLds L;
@@ -312,7 +404,8 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
   const int slot = A.slot[b], ch = (slot < 0 ? 0 : slot) * A.n_kv + kvh;
   if (split == A.nsplit) { tail_block(A, b, kvh, ch, slot); return; }
   const long qh0 = (long)b * A.n_q + (long)kvh * G;
-  build_tables(L, tid, A, ch % A.NB, qh0);
+  TableRegs Tr;
+  tables_load(Tr, tid, A, ch % A.NB, qh0);
 
   const int S = slot < 0 ? 0 : A.sl[ch];
   const int ntiles = (S + T - 1) / T, chunk = (ntiles + A.nsplit - 1) / A.nsplit;
@@ -339,6 +432,7 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
     load_tile(B, t0, lane, Tg, R0);
     load_tags(B, min(t0 + 4, tlast), a, Tg);
   }
+  tables_store(L, Tr, tid);
   __syncthreads();        // block tables are ready
   // Q as the B operand of the score product: lane (head a, quad q), product u covers group 4q+u in word order (e, e+4);
   // exponent-base words of the lane's units
@@ -359,27 +453,27 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
       TgC1 = Tg;
       load_tile(B, t + 4, lane, Tg, R1);
       load_tags(B, min(t + 8, tlast), a, Tg);
-      consume_tile<false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+      consume<false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
       TgC0 = Tg;
       load_tile(B, t + 8, lane, Tg, R0);
       load_tags(B, min(t + 12, tlast), a, Tg);
-      consume_tile<false>(R1, st, L, B, TgC1.kto, TgC1.vto, t + 4, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+      consume<false>(R1, st, L, B, TgC1.kto, TgC1.vto, t + 4, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
     }
     const int t = t0 + 4 * i;
     if (n - i == 2) {
       TgC1 = Tg;
       load_tile(B, t + 4, lane, Tg, R1);
-      consume_tile<false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
-      consume_tile<false>(R1, st, L, B, TgC1.kto, TgC1.vto, t + 4, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+      consume<false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+      consume<false>(R1, st, L, B, TgC1.kto, TgC1.vto, t + 4, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
     } else {
-      consume_tile<false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+      consume<false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
     }
   }
   if (own_partial) {
     const int t = ntiles - 1;
     load_tags(B, t, a, Tg);
     load_tile(B, t, lane, Tg, R0);
-    consume_tile<true>(R0, st, L, B, Tg.kto, Tg.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+    consume<true>(R0, st, L, B, Tg.kto, Tg.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
   }
   // The accumulators are MFMA results: keep their first non-MFMA read a full MFMA latency away on every path.
   asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");
@@ -408,9 +502,10 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
       Lc += L.l[w][g] * f; Ac += L.acc[w][g][d] * f;
     }
     const long pidx = (qh0 + g) * A.nslot + split;
-    if (d == 0) { A.pm[pidx] = M; A.pl[pidx] = Lc; }
-    A.pa[pidx * D + d] = Ac;
+    if (d == 0) { store_partial(A.pm + pidx, M); store_partial(A.pl + pidx, Lc); }
+    store_partial(A.pa + pidx * D + d, Ac);
   }
+  publish_and_merge(A, bh, qh0, G, tid);
 }
 
 // ---------------------------------------------------------------------------------------------------- split merge
@@ -464,7 +559,7 @@ static int attn_split_impl(
     const uint8_t* smk, const uint8_t* ck, const int* fk, const int* tok, const uint8_t* ovk, const int* ohsk, const uint8_t* b3k, const uint8_t* b4k,
     const uint8_t* smv, const uint8_t* cv, const int* fv, const int* tov, const uint8_t* ovv, const int* ohsv, const uint8_t* b3v, const uint8_t* b4v,
     const void* q, const int* slot, int B, int n_q, int n_kv, const int* SL, int S_pad, float scale, int nsplit, int NB,
-    const void* kt, const void* vt, const int* TL, int TCAP, float* pm, float* pl, float* pa, void* stream) {
+    const void* kt, const void* vt, const int* TL, int TCAP, float* pm, float* pl, float* pa, int* tickets, void* out, void* stream) {
   GAAC_REQUIRE(n_kv > 0 && n_q > 0 && n_q % n_kv == 0 && n_q / n_kv >= 1 && n_q / n_kv <= GMAX, "GQA group size must be 1..%d (n_q=%d, n_kv=%d)", GMAX, n_q, n_kv);
   GAAC_REQUIRE(smk && ck && fk && tok && ovk && ohsk && b3k && b4k && smv && cv && fv && tov && ovv && ohsv && b3v && b4v, "gaac_attn: null store pointer");
   GAAC_REQUIRE(q && slot && SL && pm && pl && pa, "gaac_attn: null pointer");
@@ -480,6 +575,8 @@ static int attn_split_impl(
   A.S_pad = S_pad; A.scale_log2e = scale * 1.4426950408889634f; A.nsplit = nsplit; A.nslot = nslot;
   A.n_kv = n_kv; A.n_q = n_q; A.G = n_q / n_kv; A.NB = NB;
   A.kt = (const u16*)kt; A.vt = (const u16*)vt; A.tl = TL; A.tcap = TCAP;
+  A.tickets = tickets; A.out = (u16*)out;
+  GAAC_REQUIRE(!tickets || out, "gaac_attn: the fused merge needs an output buffer");
   hipLaunchKernelGGL(k_attn_split, dim3(B * n_kv, nslot), dim3(256), 0, (hipStream_t)stream, A);
   return launch_status("gaac_attn(split)");
 }
@@ -490,7 +587,7 @@ extern "C" int gaac_attn_split(
     const void* q, const int* slot, int B, int n_q, int n_kv, const int* SL, int S_pad, float scale, int nsplit, int NB,
     const void* kt, const void* vt, const int* TL, int TCAP, float* pm, float* pl, float* pa, void* stream) {
   return attn_split_impl(smk, ck, fk, tok, ovk, ohsk, b3k, b4k, smv, cv, fv, tov, ovv, ohsv, b3v, b4v, q, slot, B, n_q, n_kv, SL, S_pad,
-                         scale, nsplit, NB, kt, vt, TL, TCAP, pm, pl, pa, stream);
+                         scale, nsplit, NB, kt, vt, TL, TCAP, pm, pl, pa, nullptr, nullptr, stream);
 }
 
 extern "C" int gaac_attn_combine(const float* pm, const float* pl, const float* pa, void* out, int n_rows, int nslot, void* stream) {
@@ -507,7 +604,18 @@ extern "C" int gaac_attn_launch(
     float* pm, float* pl, float* pa, void* out, void* stream) {
   GAAC_REQUIRE(out, "gaac_attn_launch: null output");
   int rc = attn_split_impl(smk, ck, fk, tok, ovk, ohsk, b3k, b4k, smv, cv, fv, tov, ovv, ohsv, b3v, b4v, q, slot, B, n_q, n_kv, SL, S_pad,
-                           scale, nsplit, NB, kt, vt, TL, TCAP, pm, pl, pa, stream);
+                           scale, nsplit, NB, kt, vt, TL, TCAP, pm, pl, pa, nullptr, nullptr, stream);
   if (rc) return rc;
   return gaac_attn_combine(pm, pl, pa, out, B * n_q, nsplit + (kt ? 1 : 0), stream);
+}
+
+extern "C" int gaac_attn_fused(
+    const uint8_t* smk, const uint8_t* ck, const int* fk, const int* tok, const uint8_t* ovk, const int* ohsk, const uint8_t* b3k, const uint8_t* b4k,
+    const uint8_t* smv, const uint8_t* cv, const int* fv, const int* tov, const uint8_t* ovv, const int* ohsv, const uint8_t* b3v, const uint8_t* b4v,
+    const void* q, const int* slot, int B, int n_q, int n_kv, const int* SL, int S_pad, float scale, int nsplit, int NB,
+    const void* kt, const void* vt, const int* TL, int TCAP,
+    float* pm, float* pl, float* pa, int* tickets, void* out, void* stream) {
+  GAAC_REQUIRE(out && tickets, "gaac_attn_fused: null output or ticket buffer");
+  return attn_split_impl(smk, ck, fk, tok, ovk, ohsk, b3k, b4k, smv, cv, fv, tov, ovv, ohsv, b3v, b4v, q, slot, B, n_q, n_kv, SL, S_pad,
+                         scale, nsplit, NB, kt, vt, TL, TCAP, pm, pl, pa, tickets, out, stream);
 }

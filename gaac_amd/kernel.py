@@ -1,8 +1,8 @@
 """Fused decode attention over the compressed KV on MI355X.  Public surface of /root/reference/gaac/kernel.py:332-359.
 
 attention() launches the split-K kernel (one block per (batch row, kv head, split), MFMA score and output products on
-K/V decoded in registers, optional raw-BF16 tail as one more block row) and the merge kernel, on the current stream,
-with no host synchronization.  Cache heads are addressed through a slot map exactly as in the reference: batch row b
+K/V decoded in registers, optional raw-BF16 tail as one more block row; the last block of a kv head to finish merges
+the partials) on the current stream, with no host synchronization.  Cache heads are addressed through a slot map exactly as in the reference: batch row b
 reads cache head SLOT[b]*n_kv + kvh, SLOT[b] < 0 = padded row (output 0)."""
 from __future__ import annotations
 import torch
@@ -32,6 +32,8 @@ class AttnWorkspace:
         self.pm = torch.empty(rows * nslot, dtype=torch.float32, device=dev)
         self.pl = torch.empty(rows * nslot, dtype=torch.float32, device=dev)
         self.pa = torch.empty(rows * nslot * D, dtype=torch.float32, device=dev)
+        # arrival counters of the fused merge, one per (batch row, kv head) (at most `rows` of them); every launch leaves them zero
+        self.tickets = torch.zeros(rows, dtype=torch.int32, device=dev)
 
 
 def _store_args(st):
@@ -40,9 +42,10 @@ def _store_args(st):
     return (p(st.sm), p(st.codes), p(st.flags), p(st.tile_off), p(st.ovf), p(hs), p(st.base3), p(st.base4))
 
 
-def attn_launch(K, V, q2d, slots, n_q, n_kv, SL, S_pad, scale, nsplit, kt=None, vt=None, TL=None, TCAP=0, ws=None, phase="both"):
+def attn_launch(K, V, q2d, slots, n_q, n_kv, SL, S_pad, scale, nsplit, kt=None, vt=None, TL=None, TCAP=0, ws=None, phase="fused"):
     """K, V: objects with sm, codes, flags, tile_off, ovf, head_start|ovf_head_start, base3, base4 (a Page or a cache store).
-    q2d: [B*n_q, D] bf16 contiguous.  Returns [B*n_q, D] bf16.  phase: "both" | "split" | "combine" (the halves of the launch)."""
+    q2d: [B*n_q, D] bf16 contiguous.  Returns [B*n_q, D] bf16.  phase: "fused" (one kernel, the last block of each
+    kv head merges) | "both" (split kernel then merge kernel) | "split" | "combine" (the halves of "both")."""
     G = n_q // max(1, n_kv)
     if not (1 <= G <= GMAX and G * n_kv == n_q):
         raise RuntimeError(f"GQA group size must be 1..{GMAX}")
@@ -62,14 +65,16 @@ def attn_launch(K, V, q2d, slots, n_q, n_kv, SL, S_pad, scale, nsplit, kt=None, 
     args = (*_store_args(K), *_store_args(V), p(q2d), p(slots), B, n_q, n_kv, p(SL), S_pad, float(scale), nsplit, K.base3.shape[0],
             p(kt) if has_tail else None, p(vt) if has_tail else None, p(TL) if has_tail else None, TCAP if has_tail else 0,
             p(ws.pm), p(ws.pl), p(ws.pa))
-    if phase == "split":
+    if phase == "fused":
+        _lib.call("gaac_attn_fused", *args, p(ws.tickets), p(ws.out), _lib.stream())
+    elif phase == "split":
         _lib.call("gaac_attn_split", *args, _lib.stream())
     else:
         _lib.call("gaac_attn_launch", *args, p(ws.out), _lib.stream())
     return ws.out
 
 
-def attention(q, kp, vp, scale=None, nsplit=None):
+def attention(q, kp, vp, scale=None, nsplit=None, phase="fused"):
     """Decode attention over two Pages (kinds 'k' / 'v', H = B*n_kv heads of equal length).
     q: [B, n_q, D] bf16 (one query token per sequence) -> [B, n_q, D] bf16."""
     B, n_q, Dq = q.shape
@@ -79,5 +84,5 @@ def attention(q, kp, vp, scale=None, nsplit=None):
     slots = torch.arange(B, dtype=torch.int32, device=dev)
     SL = torch.full((kp.H,), kp.S, dtype=torch.int32, device=dev)
     out = attn_launch(kp, vp, q.reshape(B * n_q, Dq).contiguous(), slots, n_q, n_kv, SL, kp.sm.shape[1] // D,
-                      scale if scale is not None else Dq ** -0.5, nsplit)
+                      scale if scale is not None else Dq ** -0.5, nsplit, phase=phase)
     return out.view(B, n_q, Dq)

@@ -72,6 +72,17 @@ int gaac_attn_split(
     const void* kt, const void* vt, const int* TL, int TCAP, float* pm, float* pl, float* pa, void* stream);
 int gaac_attn_combine(const float* pm, const float* pl, const float* pa, void* out, int n_rows, int nslot, void* stream);
 
+/* gaac_attn_launch as ONE kernel: every block publishes its partial and draws a ticket from tickets[b*n_kv + kv head];
+ * the block that draws the last one merges the NSLOT partials of its G query heads (gaac_combine, kernel.py:281-294) and
+ * resets the counter.  tickets: int32 [B*n_kv], zero before the first launch (each launch leaves it zero); launches that
+ * share pm/pl/pa/tickets must be ordered on one stream. */
+int gaac_attn_fused(
+    const uint8_t* smk, const uint8_t* ck, const int* fk, const int* tok, const uint8_t* ovk, const int* ohsk, const uint8_t* b3k, const uint8_t* b4k,
+    const uint8_t* smv, const uint8_t* cv, const int* fv, const int* tov, const uint8_t* ovv, const int* ohsv, const uint8_t* b3v, const uint8_t* b4v,
+    const void* q, const int* slot, int B, int n_q, int n_kv, const int* SL, int S_pad, float scale, int nsplit, int NB,
+    const void* kt, const void* vt, const int* TL, int TCAP,
+    float* pm, float* pl, float* pa, int* tickets, void* out, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -54,6 +54,26 @@ def test_result_does_not_depend_on_the_split_count():
         assert np.abs(o - outs[0]).max() <= 2 ** -7 * np.abs(outs[0]).max()
 
 
+def test_fused_merge_equals_the_two_kernel_launch_and_rearms_its_tickets():
+    """One-kernel launch (last block merges) vs split kernel + merge kernel: same partials, so the outputs agree to the last
+    bf16 bit or one ulp of rounding order; launched three times on one workspace to show the counters reset themselves."""
+    dev = require_gpu()
+    from gaac_amd.kernel import attn_launch, AttnWorkspace
+    for (B, n_kv, G, S, ns) in [(1, 8, 4, 4096, 16), (2, 2, 16, 1000, 7), (3, 2, 1, 16, 1), (1, 8, 4, 8192, 64)]:
+        _, _, kp, vp = _pages(B, n_kv, S, dev)
+        n_q = n_kv * G
+        q = to_bf16(randn_bf16((B * n_q, 128), seed=9, scale=0.3), dev)
+        slots = torch.arange(B, dtype=torch.int32, device=dev)
+        SL = torch.full((B * n_kv,), S, dtype=torch.int32, device=dev)
+        ws = AttnWorkspace(B * n_q, ns, torch.bfloat16, dev)
+        run = lambda ph: attn_launch(kp, vp, q, slots, n_q, n_kv, SL, kp.sm.shape[1] // 128, SCALE, ns, ws=ws, phase=ph).float().clone()
+        two = run("both")
+        for _ in range(3):
+            one = run("fused")
+            assert (one - two).abs().max().item() <= 2.0 ** -7 * two.abs().max().item()
+        assert int(ws.tickets.abs().sum().item()) == 0
+
+
 def test_stated_tolerance_on_unit_scale_data():
     """max-abs <= 1e-2 and mean-abs <= 1e-3 against decompress + fp32 softmax attention, q ~ N(0,1)."""
     dev = require_gpu()
