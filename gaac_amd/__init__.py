@@ -3,5 +3,6 @@ slot cache) for AMD MI355X, with the Python surface of the reference's `gaac` pa
 from .codec import Codec, Page
 from .encoder import TileEncoder
 from .kernel import attention, choose_nsplit
+from .kv_cache import CompressedKVCache
 
-__all__ = ["Codec", "Page", "TileEncoder", "attention", "choose_nsplit"]
+__all__ = ["Codec", "Page", "TileEncoder", "attention", "choose_nsplit", "CompressedKVCache"]

@@ -31,9 +31,15 @@ __device__ __forceinline__ void stage_bases(EncodeLds& L, const uint8_t* __restr
   if (lane < T) L.tags[lane] = 0u;
 }
 
+// Orders the LDS traffic of ONE wave (LDS operations of a wave complete in program order; the fences only stop the compiler from
+// moving them): what any lane wrote before is visible to every lane of the same wave after.
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 // Encodes the tile staged in L (after a barrier).  Writes the native sign/mantissa and code bytes, the 16 tag words (one per line) and
 // the escape bytes (at esc_dst + offset-in-tile; nullptr = count only).  Returns the tile's escape byte count (all lanes).
-// Must be called by all 64 lanes of a one-wave block: it uses block barriers.
+// Must be called by all 64 lanes of the wave that owns L; it synchronises that wave only.
 template <int KIND>
 __device__ __forceinline__ int encode_staged_tile(EncodeLds& L, int nvalid, int lane, uint8_t* __restrict__ sm_tile,
                                                   uint8_t* __restrict__ cd_tile, int* __restrict__ flags_tile,
@@ -75,13 +81,13 @@ __device__ __forceinline__ int encode_staged_tile(EncodeLds& L, int nvalid, int 
   *reinterpret_cast<u32*>(cd_tile + 4 * lane) = g24[0] | (g24[1] << 24);
   *reinterpret_cast<u32*>(cd_tile + 256 + 4 * lane) = (g24[1] >> 8) | (g24[2] << 16);
   *reinterpret_cast<u32*>(cd_tile + 512 + 4 * lane) = (g24[2] >> 16) | (g24[3] << 8);
-  __syncthreads();
+  wave_lds_sync();
   {
     const u32 f = L.tags[a];
     const u32 rb = (u32)esc_bytes(f), incl = row_scan16(rb);
     if (lane < T) { L.rowoff[lane] = (int)(incl - rb); flags_tile[lane] = (int)f; if (lane == T - 1) L.rowoff[T] = (int)incl; }
   }
-  __syncthreads();
+  wave_lds_sync();
   if (esc_dst) {
     uint8_t* p = esc_dst + L.rowoff[a] + esc_prefix(L.tags[a], 8 * q);
 #pragma unroll

@@ -26,9 +26,9 @@ def choose_nsplit(B: int, n_kv: int, S: int, target_ctas: int = 512, min_tok: in
 
 class AttnWorkspace:
     """Output + split partials of one launch shape (fp32 m, l [rows*NSLOT] and acc [rows*NSLOT*D]; rows = B*n_q)."""
-    def __init__(self, rows: int, nslot: int, dtype, dev):
+    def __init__(self, rows: int, nslot: int, dtype, dev, with_out: bool = True):
         self.rows, self.nslot = rows, nslot
-        self.out = torch.empty(rows, D, dtype=dtype, device=dev)
+        self.out = torch.empty(rows, D, dtype=dtype, device=dev) if with_out else None      # None: a fresh output per launch
         self.pm = torch.empty(rows * nslot, dtype=torch.float32, device=dev)
         self.pl = torch.empty(rows * nslot, dtype=torch.float32, device=dev)
         self.pa = torch.empty(rows * nslot * D, dtype=torch.float32, device=dev)
@@ -59,19 +59,20 @@ def attn_launch(K, V, q2d, slots, n_q, n_kv, SL, S_pad, scale, nsplit, kt=None, 
     elif ws.rows != B * n_q or ws.nslot != nslot:
         raise RuntimeError("attention workspace does not match the launch shape")
     p = _lib.ptr
+    out = ws.out if ws.out is not None else torch.empty(B * n_q, D, dtype=q2d.dtype, device=q2d.device)
     if phase == "combine":
-        _lib.call("gaac_attn_combine", p(ws.pm), p(ws.pl), p(ws.pa), p(ws.out), B * n_q, nslot, _lib.stream())
-        return ws.out
+        _lib.call("gaac_attn_combine", p(ws.pm), p(ws.pl), p(ws.pa), p(out), B * n_q, nslot, _lib.stream())
+        return out
     args = (*_store_args(K), *_store_args(V), p(q2d), p(slots), B, n_q, n_kv, p(SL), S_pad, float(scale), nsplit, K.base3.shape[0],
             p(kt) if has_tail else None, p(vt) if has_tail else None, p(TL) if has_tail else None, TCAP if has_tail else 0,
             p(ws.pm), p(ws.pl), p(ws.pa))
     if phase == "fused":
-        _lib.call("gaac_attn_fused", *args, p(ws.tickets), p(ws.out), _lib.stream())
+        _lib.call("gaac_attn_fused", *args, p(ws.tickets), p(out), _lib.stream())
     elif phase == "split":
         _lib.call("gaac_attn_split", *args, _lib.stream())
     else:
-        _lib.call("gaac_attn_launch", *args, p(ws.out), _lib.stream())
-    return ws.out
+        _lib.call("gaac_attn_launch", *args, p(out), _lib.stream())
+    return out
 
 
 def attention(q, kp, vp, scale=None, nsplit=None, phase="fused"):

@@ -83,6 +83,19 @@ int gaac_attn_fused(
     const void* kt, const void* vt, const int* TL, int TCAP,
     float* pm, float* pl, float* pa, int* tickets, void* out, void* stream);
 
+/* CompressedKVCache.append, /root/reference/gaac/kv_cache.py:172-181 (kernels _append_one/_append_kv/_advance, :22-96), as one
+ * launch: row i = b*n_kv + kvh of k_new/v_new [B, n_kv, 128] bf16 goes to tail row tail_len[h] of cache head
+ * h = slots[b]*n_kv + kvh (slots[b] < 0: skipped); when that fills the 16-row tail the tile is compressed in place as tile S[h]/16
+ * (token stride cap), its escape bytes are appended at ovf + h*ovf_cap + ovf_used[h], and tile_off, ovf_used, tail_len and S advance.
+ * Per kind: tail bf16 [H,16,128], base3/base4 u8 [NB,128] (row h % NB), sm u8 [H,cap*128], codes u8 [H,cap*48], flags i32 [H,cap],
+ * ovf u8 [H*ovf_cap], tile_off i32 [H,cap/16], ovf_used i32 [H].  Instead of writing out of bounds the kernel ORs into *err:
+ * 1 = a head was at capacity (token dropped), 2 = an escape stream was full (tile stored with zero tags). */
+int gaac_cache_append(
+    const int* slots, int B, int n_kv, const void* k_new, const void* v_new, int* tail_len, int* S, int cap, int ovf_cap, int NB,
+    void* k_tail, const uint8_t* k_base3, const uint8_t* k_base4, uint8_t* k_sm, uint8_t* k_codes, int* k_flags, uint8_t* k_ovf, int* k_tile_off, int* k_ovf_used,
+    void* v_tail, const uint8_t* v_base3, const uint8_t* v_base4, uint8_t* v_sm, uint8_t* v_codes, int* v_flags, uint8_t* v_ovf, int* v_tile_off, int* v_ovf_used,
+    int* err, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

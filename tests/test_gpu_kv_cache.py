@@ -1,0 +1,133 @@
+"""GPU tests of the slot cache: prefill / append / attention / decompress over a changing batch and one decode step replayed
+as a HIP graph.  Same scenarios and tolerances as /root/reference/tests/test_kv_cache.py:15-86; the expected values come
+from the history kept on the host (bit-exact decompress) and the oracle's fp32 attention."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gaac_oracle as O
+from common import kv_like16, to_bf16, to_u16, randn_bf16
+from gpu_util import require_gpu
+
+pytestmark = pytest.mark.gpu
+N_KV, G, SCALE = 4, 4, 128 ** -0.5
+
+
+def _tok16(x16):          # [n_kv, L, D] -> token-major [L, n_kv, D]
+    return np.ascontiguousarray(x16.transpose(1, 0, 2))
+
+
+def _bases(seed, dev):
+    from gaac_amd.codec import exponent_hist, bases_from_hist
+    out = {}
+    for name, sd in (("k", seed), ("v", seed + 1)):
+        x = to_bf16(_tok16(kv_like16(N_KV, 4096, seed=sd, scale_seed=1000 + (name == "v"))), dev)
+        out[name + "3"], out[name + "4"] = bases_from_hist(exponent_hist(x, N_KV), N_KV)
+    return out
+
+
+def _prompt(L, seed):
+    return _tok16(kv_like16(N_KV, L, seed=seed, scale_seed=1000)), _tok16(kv_like16(N_KV, L, seed=seed + 500, scale_seed=1001))
+
+
+def _check(cache, hist, slots_l, q16, dev):
+    slots = torch.tensor(slots_l, dtype=torch.int32, device=dev)
+    out = O.bf16_to_f32(to_u16(cache.attention(to_bf16(q16, dev), slots, SCALE)))
+    for b, s in enumerate(slots_l):
+        if s < 0:
+            assert np.abs(out[b]).max() == 0
+            continue
+        k16, v16 = hist[s]
+        ref = O.ref_attention(q16[b], k16, v16, SCALE)
+        assert np.abs(out[b] - ref).max() <= 2e-2 * np.abs(ref).max() + 1e-3
+        dk, dv = cache.decompress(s)
+        assert np.array_equal(to_u16(dk), k16) and np.array_equal(to_u16(dv), v16)
+
+
+@pytest.mark.parametrize("static_bases", [True, False])
+def test_slots_prefill_append(static_bases):
+    dev = require_gpu()
+    from gaac_amd import CompressedKVCache
+    cache = CompressedKVCache(n_slots=4, n_kv=N_KV, capacity=1024, bases=_bases(10, dev) if static_bases else None)
+    hist = {}
+    for s, L in {0: 37, 2: 500, 3: 16}.items():
+        k16, v16 = _prompt(L, 20 + s)
+        cache.prefill(s, to_bf16(k16, dev), to_bf16(v16, dev)); hist[s] = (k16, v16)
+    for step in range(40):      # decode steps over a changing batch (slot order != batch order, plus a padded row)
+        slots_l = [3, 0, 2, -1] if step % 3 else [2, 3, -1, 0]
+        k16 = randn_bf16((4, N_KV, 128), seed=100 + step, scale=0.5); v16 = randn_bf16((4, N_KV, 128), seed=200 + step, scale=0.5)
+        cache.append(torch.tensor(slots_l, dtype=torch.int32, device=dev), to_bf16(k16, dev), to_bf16(v16, dev))
+        for b, s in enumerate(slots_l):
+            if s >= 0: hist[s] = (np.concatenate([hist[s][0], k16[b:b + 1]]), np.concatenate([hist[s][1], v16[b:b + 1]]))
+        if step % 16 == 15: cache.check_capacity()
+        if step % 13 == 0 or step == 39:
+            _check(cache, hist, slots_l, randn_bf16((4, N_KV * G, 128), seed=300 + step, scale=0.1), dev)
+    st = cache.stats()
+    assert st["tokens"] == sum(len(h[0]) for h in hist.values())
+    S = sum(len(h[0]) // 16 * 16 for h in hist.values()) * N_KV; tl = sum(len(h[0]) % 16 for h in hist.values()) * N_KV
+    esc = int(cache.k.ovf_used.sum()) + int(cache.v.ovf_used.sum())
+    assert st["bytes_used"] == 2 * (S * 180 + S // 16 * 4 + tl * 256) + esc and st["bf16_bytes"] == 2 * (S + tl) * 256
+    # slot reuse: a new sequence replaces slot 0
+    k16, v16 = _prompt(64, 99)
+    cache.prefill(0, to_bf16(k16, dev), to_bf16(v16, dev)); hist[0] = (k16, v16)
+    _check(cache, hist, [0], randn_bf16((1, N_KV * G, 128), seed=400, scale=0.1), dev)
+
+
+def test_graph_decode_step():
+    """append + attention captured once and replayed 40 times (two tails fill up on the way), every replay checked."""
+    dev = require_gpu()
+    from gaac_amd import CompressedKVCache
+    cache = CompressedKVCache(n_slots=2, n_kv=N_KV, capacity=512, bases=_bases(11, dev))
+    k0, v0 = _prompt(200, 5)
+    cache.prefill(1, to_bf16(k0, dev), to_bf16(v0, dev))
+    slots = torch.tensor([1, -1], dtype=torch.int32, device=dev)
+    q = torch.zeros(2, N_KV * G, 128, dtype=torch.bfloat16, device=dev)
+    kn = torch.zeros(2, N_KV, 128, dtype=torch.bfloat16, device=dev); vn = torch.zeros_like(kn)
+    def step():
+        cache.append(slots, kn, vn); return cache.attention(q, slots, SCALE, max_len=512)
+    s = torch.cuda.Stream(); s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):          # warm up outside capture with every row padded (nothing is appended)
+        slots.fill_(-1); step()
+    torch.cuda.current_stream().wait_stream(s)
+    cache.growable = False
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        out = step()
+    slots.copy_(torch.tensor([1, -1], dtype=torch.int32))
+    hk, hv = k0, v0
+    for i in range(40):
+        k16 = randn_bf16((2, N_KV, 128), seed=500 + i, scale=0.5); v16 = randn_bf16((2, N_KV, 128), seed=600 + i, scale=0.5)
+        q16 = randn_bf16((2, N_KV * G, 128), seed=700 + i, scale=0.1)
+        kn.copy_(to_bf16(k16, dev)); vn.copy_(to_bf16(v16, dev)); q.copy_(to_bf16(q16, dev))
+        g.replay(); torch.cuda.synchronize()
+        hk, hv = np.concatenate([hk, k16[:1]]), np.concatenate([hv, v16[:1]])
+        got = O.bf16_to_f32(to_u16(out))
+        ref = O.ref_attention(q16[0], hk, hv, SCALE)
+        assert np.abs(got[0] - ref).max() <= 2e-2 * np.abs(ref).max() + 1e-3, i
+        assert np.abs(got[1]).max() == 0
+    dk, dv = cache.decompress(1)
+    assert np.array_equal(to_u16(dk), hk) and np.array_equal(to_u16(dv), hv)
+    cache.check_capacity()
+
+
+def test_overflow_is_flagged_not_written():
+    """A head at capacity drops the token and raises at the next check; an escape stream without room stores a zero-tagged tile."""
+    dev = require_gpu()
+    from gaac_amd import CompressedKVCache
+    cache = CompressedKVCache(n_slots=1, n_kv=N_KV, capacity=32, bases=_bases(12, dev))
+    k16, v16 = _prompt(32, 7)
+    cache.prefill(0, to_bf16(k16, dev), to_bf16(v16, dev))
+    slots = torch.zeros(1, dtype=torch.int32, device=dev)
+    for i in range(16):
+        cache.append(slots, to_bf16(randn_bf16((1, N_KV, 128), seed=i), dev), to_bf16(randn_bf16((1, N_KV, 128), seed=50 + i), dev))
+    assert int(cache.S.max()) == 32 and int(cache.tail_len.max()) == 0
+    with pytest.raises(RuntimeError, match="token capacity"):
+        cache.check_capacity()
+    # escape stream: all-raw tiles (exponents far from the bases) need 1280 B per tile, the stream holds 2*16+8
+    cache = CompressedKVCache(n_slots=1, n_kv=N_KV, capacity=64, bases=_bases(12, dev), ovf_bytes_per_tile=8)
+    cache.growable = False
+    big = to_bf16(np.full((1, N_KV, 128), 0x7F00, dtype=np.uint16), dev)
+    for i in range(16): cache.append(slots, big, big)
+    with pytest.raises(RuntimeError, match="escape stream"):
+        cache.check_capacity()
+    assert int(cache.k.ovf_used.max()) == 0 and int(cache.k.flags.abs().max()) == 0
