@@ -2,7 +2,8 @@
 
   python bench.py [--gpus 1] [--steps K] [--warmup W]
 
-A step = one layer's decode attention (split pass incl. the 7-token BF16 tail + merge) for config 1 of BASELINE.json:
+A step = one layer's decode attention (ONE kernel: split pass incl. the 7-token BF16 tail, merged by the last block of each
+kv head) for config 1 of BASELINE.json:
 32 query heads over 8 kv heads (GQA group 4), head_dim 128, 65536 compressed tokens + 7 tail tokens, batch 1.
 Inputs are synthetic (seeded, CPU generator), encoded once with the HIP encoder and resident in HBM before timing.
 Successive steps rotate over distinct copies of the compressed KV so the 256 MB Infinity Cache cannot serve them.
@@ -49,7 +50,7 @@ def clone_store(page):
     return c
 
 
-def cpu_baseline(k16: np.ndarray, v16: np.ndarray, q16: np.ndarray, b3k, b4k, b3v, b4v, scale: float, heads: int) -> dict:
+def cpu_baseline(k16: np.ndarray, v16: np.ndarray, q16: np.ndarray, b3k, b4k, b3v, b4v, scale: float, heads: int, reps: int = 4) -> dict:
     """The CPU oracle's decompress + fp32 softmax attention on `heads` kv heads of the same workload (bounded sample),
     timed on this box's host cores; pages are encoded beforehand (not timed)."""
     from oracle import gaac_oracle as O
@@ -58,21 +59,22 @@ def cpu_baseline(k16: np.ndarray, v16: np.ndarray, q16: np.ndarray, b3k, b4k, b3
     vp = O.encode(v16[:heads], "v", b3v[:heads], b4v[:heads], heads)
     with threadpool_limits(limits=1):
         t0 = time.perf_counter()
-        kd, vd = O.decode(kp), O.decode(vp)
-        out = O.ref_attention(q16[:heads * G], kd.transpose(1, 0, 2), vd.transpose(1, 0, 2), scale)
-        dt = time.perf_counter() - t0
+        for _ in range(reps):
+            kd, vd = O.decode(kp), O.decode(vp)
+            out = O.ref_attention(q16[:heads * G], kd.transpose(1, 0, 2), vd.transpose(1, 0, 2), scale)
+        dt = (time.perf_counter() - t0) / reps
     assert np.array_equal(kd, k16[:heads]) and np.array_equal(vd, v16[:heads]) and np.isfinite(out).all()
     us_layer = dt * 1e6 * (N_KV / heads)
     return {"value": us_layer, "unit": "us/layer", "cores": 1, "kind": "port",
             "sample": f"{heads} of {N_KV} kv heads x {k16.shape[1]} tokens (K and V): numpy oracle decode + fp32 softmax attention, "
-                      f"{dt:.1f} s measured, scaled x{N_KV // heads}; host has {os.cpu_count()} cpus"}
+                      f"mean of {reps} passes of {dt:.1f} s, scaled x{N_KV / heads:g}; host has {os.cpu_count()} cpus, 1 thread used"}
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1); ap.add_argument("--steps", type=int, default=300); ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--copies", type=int, default=3); ap.add_argument("--nsplit", type=int, default=0)
-    ap.add_argument("--cpu-heads", type=int, default=1, help="kv heads in the CPU baseline sample (0 = skip)")
+    ap.add_argument("--cpu-heads", type=int, default=8, help="kv heads in the CPU baseline sample (0 = skip)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one MI355X; this build has no multi-GPU path (the hot path shards by kv head without any exchange). Use --gpus 1.", file=sys.stderr)
@@ -104,7 +106,7 @@ def main():
     alg_bytes = kp.nbytes + vp.nbytes + 2 * N_KV * TAIL_TOK * D * 2 + 2 * n_q * D * 2 + 4 * N_KV * D
     bf16_bytes = 2 * H * (S_CTX + TAIL_TOK) * D * 2 + 2 * n_q * D * 2
 
-    def step(i, phase="both"):
+    def step(i, phase="fused"):
         K, V = pages[i % len(pages)]
         return attn_launch(K, V, q2d, slots, n_q, N_KV, SL, S_pad, scale, nsplit, kt, vt, TL, 16, ws=ws, phase=phase)
 
@@ -135,12 +137,17 @@ def main():
     dt = time.perf_counter() - t0
     us_step = dt * 1e6 / a.steps
 
-    # ---- per-kernel duration of the split pass (the dominant kernel): HIP events on the launch stream, eager launches
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(a.steps)]
-    for i in range(a.steps):
-        evs[i][0].record(); step(i, "split"); evs[i][1].record(); step(i, "combine")
+    # ---- duration of the attention kernel itself: HIP events on the launch stream around batches of back-to-back launches
+    # (one event pair per launch would add the event's own ~3 us to every sample)
+    BATCH = 20
+    nb = max(5, a.steps // BATCH)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nb)]
+    for b_, (e0, e1) in enumerate(evs):
+        e0.record()
+        for i in range(BATCH): step(b_ * BATCH + i)
+        e1.record()
     torch.cuda.synchronize()
-    ts = sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in evs)
+    ts = sorted(e0.elapsed_time(e1) * 1e3 / BATCH for e0, e1 in evs)
     split_us_mean, split_us_med = sum(ts) / len(ts), ts[len(ts) // 2]
 
     # ---- uncompressed BF16 decode attention on the same GPU (torch SDPA over the same tokens), rotating copies
@@ -171,7 +178,7 @@ def main():
         "bf16_sdpa_us": round(bf16_us, 2), "speedup_vs_bf16_sdpa": round(bf16_us / us_step, 3),
         "roofline": {"bound": "hbm", "achieved": round(alg_bytes / split_us_mean / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(alg_bytes / split_us_mean / 1e3 / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "k_attn_split", "kernel_us_mean": round(split_us_mean, 2), "kernel_us_median": round(split_us_med, 2)},
+                     "kernel": "k_attn_split (split pass + tail + fused merge)", "kernel_us_mean": round(split_us_mean, 2), "kernel_us_median": round(split_us_med, 2)},
     }
     if a.cpu_heads > 0:
         b = lambda t: t.cpu().numpy()
