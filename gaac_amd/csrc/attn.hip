@@ -47,39 +47,58 @@ __device__ __forceinline__ u32 pack_bf16x2(float lo, float hi) {
 // agent-scope accesses (write-through stores, cache-bypassing loads) instead of whole-L2 write-back/invalidate fences.
 typedef __attribute__((ext_vector_type(4))) float f32x4v;
 __device__ __forceinline__ void store_partial(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-__device__ __forceinline__ float load_partial(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 constexpr int AUX_AGENT_SCOPE = 0x10;      // sc1 of the gfx94x/gfx950 buffer cache policy
 __device__ __forceinline__ void merge_head_by_wave(const AttnArgs& A, long row, float* __restrict__ fs, int lane) {
+  // The m/l loads and the first 32 partial rows are issued before the first result is needed (one memory round trip for them).
+  // Buffer loads past the end of a row's partials return zero without a branch.
   const int nslot = A.nslot;
-  const float* pm = A.pm + row * nslot; const float* pl = A.pl + row * nslot;
-  const float* pa = A.pa + row * nslot * D;
+  const __amdgpu_buffer_rsrc_t rm = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(A.pm + row * nslot), 0, nslot * 4, 0x00027000);
+  const __amdgpu_buffer_rsrc_t rl = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(A.pl + row * nslot), 0, nslot * 4, 0x00027000);
+  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(A.pa + row * nslot * D), 0, nslot * D * 4, 0x00027000);
+  constexpr int PER = MAX_SLOTS / 64, CH = 16;
+  const int sg = lane >> 5, dq = (lane & 31) * 4;      // two slots per wave-wide load, four dims per lane
+  u32 mv[PER], lv[PER];
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    mv[k] = __builtin_amdgcn_raw_buffer_load_b32(rm, (lane + 64 * k) * 4, 0, AUX_AGENT_SCOPE);
+    lv[k] = __builtin_amdgcn_raw_buffer_load_b32(rl, (lane + 64 * k) * 4, 0, AUX_AGENT_SCOPE);
+  }
+  u32x4 v[CH];
+#pragma unroll
+  for (int k = 0; k < CH; ++k) v[k] = __builtin_amdgcn_raw_buffer_load_b128(ra, ((sg + 2 * k) * D + dq) * 4, 0, AUX_AGENT_SCOPE);
   float m = -INFINITY;
-  for (int s = lane; s < nslot; s += 64) m = fmaxf(m, load_partial(pm + s));
+#pragma unroll
+  for (int k = 0; k < PER; ++k) m = fmaxf(m, lane + 64 * k < nslot ? __uint_as_float(mv[k]) : -INFINITY);
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
   float l = 0.f;
-  for (int s = lane; s < nslot; s += 64) {
-    const float v = load_partial(pm + s);
-    const float f = v == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(v - m);
-    fs[s] = f; l += load_partial(pl + s) * f;
+#pragma unroll
+  for (int k = 0; k < PER; ++k) {
+    const int s = lane + 64 * k;
+    const float pmv = __uint_as_float(mv[k]);
+    const float f = (s < nslot && pmv != -INFINITY) ? __builtin_amdgcn_exp2f(pmv - m) : 0.f;
+    if (s < nslot) fs[s] = f;
+    l += __uint_as_float(lv[k]) * f;
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o, 64);
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-  const int sg = lane >> 5, dq = (lane & 31) * 4;      // two slots per wave-wide load, four dims per lane
-  const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(pa), 0, nslot * D * 4, 0x00027000);
+  wave_lds_sync();
   f32x4v acc = {0.f, 0.f, 0.f, 0.f};
-  constexpr int CH = 16;
-  for (int s0 = sg; s0 < nslot; s0 += 2 * CH) {
-    u32x4 v[CH];
 #pragma unroll
-    for (int k = 0; k < CH; ++k)      // slots past the end are out of the buffer's range and read as zero
-      v[k] = __builtin_amdgcn_raw_buffer_load_b128(rs, ((s0 + 2 * k) * D + dq) * 4, 0, AUX_AGENT_SCOPE);
+  for (int k = 0; k < CH; ++k) {
+    const int s = sg + 2 * k; const float f = s < nslot ? fs[s] : 0.f;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[c] += __uint_as_float(v[k][c]) * f;
+  }
+  for (int s0 = sg + 2 * CH; s0 < nslot; s0 += 2 * CH) {
+    u32x4 w[CH];
+#pragma unroll
+    for (int k = 0; k < CH; ++k) w[k] = __builtin_amdgcn_raw_buffer_load_b128(ra, ((s0 + 2 * k) * D + dq) * 4, 0, AUX_AGENT_SCOPE);
 #pragma unroll
     for (int k = 0; k < CH; ++k) {
       const int s = s0 + 2 * k; const float f = s < nslot ? fs[s] : 0.f;
 #pragma unroll
-      for (int c = 0; c < 4; ++c) acc[c] += __uint_as_float(v[k][c]) * f;
+      for (int c = 0; c < 4; ++c) acc[c] += __uint_as_float(w[k][c]) * f;
     }
   }
 #pragma unroll

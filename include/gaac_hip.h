@@ -96,6 +96,10 @@ int gaac_cache_append(
     void* v_tail, const uint8_t* v_base3, const uint8_t* v_base4, uint8_t* v_sm, uint8_t* v_codes, int* v_flags, uint8_t* v_ovf, int* v_tile_off, int* v_ovf_used,
     int* err, void* stream);
 
+/* Measurement aid with no counterpart in the reference: a plain copy of nbytes (multiple of 16) with 16-byte accesses per lane,
+ * the known-size kernel that HBM traffic counters (FETCH_SIZE / WRITE_SIZE) are scaled against. */
+int gaac_stream_copy(const void* src, void* dst, long nbytes, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
