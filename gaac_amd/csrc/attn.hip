@@ -8,8 +8,9 @@
 //     The score tile lands in the register layout the second product wants for P^T, so P never crosses lanes.
 //   * the GQA group (<= 16 query heads) rides in the N dimension; register use does not depend on it;
 //   * three-stage prefetch per wave: tag words of tile t+8, payload + escape bytes of tile t+4, consume tile t;
-//   * the tail (<= 16 raw BF16 tokens per head) is one extra block row of the same launch; its partial goes to the
-//     last partial slot.  Softmax runs in base 2 (scale * log2 e folded into the scores).
+//   * rows that are not compressed (the raw BF16 tail of a cache head, <= 16 tokens) are one extra block row of the same launch
+//     (dispatched first): a block without tiles whose fifth block-merge partial holds the tail; it writes partial slot nsplit.  Softmax runs in base 2 (scale * log2 e
+//     folded into the scores).
 #include "gaac_tile.h"
 #include "gaac_capi.h"
 #include "../../include/gaac_hip.h"
@@ -110,8 +111,8 @@ __device__ __forceinline__ void merge_head_by_wave(const AttnArgs& A, long row, 
   }
 }
 // Called by all 256 threads of a block after its partial has been written with store_partial().
-__device__ __forceinline__ void publish_and_merge(const AttnArgs& A, int bh, long qh0, int G, int tid) {
-  __shared__ float fs[4][MAX_SLOTS];
+// fs: 4 x MAX_SLOTS floats of LDS that nothing else uses any more.
+__device__ __forceinline__ void publish_and_merge(const AttnArgs& A, int bh, long qh0, int G, int tid, float* __restrict__ fs) {
   __shared__ int last;
   if (!A.tickets) return;
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // this thread's write-through stores have reached device scope
@@ -120,61 +121,71 @@ __device__ __forceinline__ void publish_and_merge(const AttnArgs& A, int bh, lon
   __syncthreads();
   if (!last) return;
   const int wave = tid >> 6, lane = tid & 63;
-  for (int g = wave; g < G; g += 4) merge_head_by_wave(A, qh0 + g, fs[wave], lane);
+  for (int g = wave; g < G; g += 4) merge_head_by_wave(A, qh0 + g, fs + wave * MAX_SLOTS, lane);
   if (tid == 0) __hip_atomic_store(&A.tickets[bh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);      // re-arm for the next launch
 }
 
-// ---------------------------------------------------------------------------------------------------- raw tail block
-__device__ void tail_block(const AttnArgs& A, int b, int kvh, int ch, int slot) {
-  __shared__ float qs[GMAX][D];
-  __shared__ float sc[GMAX][T];
-  const int tid = threadIdx.x, G = A.G;
-  const int TL = slot < 0 ? 0 : min(A.tl[ch], A.tcap);
-  const long qh0 = (long)b * A.n_q + (long)kvh * G;
-  for (int i = tid; i < G * D; i += 256) qs[i >> 7][i & 127] = bf16_bits_to_float(A.q[qh0 * D + i]);
-  __syncthreads();
+// ---------------------------------------------------------------------------------------------------- uncompressed rows
+// Attention of the block's G query heads over up to 16 rows kept as plain BF16 (the raw tail of a cache head, gaac_tail of
+// /root/reference/gaac/kernel.py:220-279), done by all 256 threads in fp32 on the VALU.  The result is folded into the running
+// partial (m, l, acc) that the block merge treats as a fifth wave; several calls accumulate (online softmax).
+struct RawScratch {              // lives in the block-merge buffer, which is idle until the waves have finished their tiles
+  float qs[GMAX][D];             // the query heads in fp32, natural channel order
+  float sc[GMAX][T];             // scores, then probabilities
+  float alpha[GMAX];             // rescale factor of the running partial
+};
+__device__ __forceinline__ void raw_rows_begin(RawScratch& R, const AttnArgs& A, long qh0, int G, int tid) {
+  for (int i = tid; i < G * D; i += 256) R.qs[i >> 7][i & 127] = bf16_bits_to_float(A.q[qh0 * D + i]);
+}
+// krows / vrows: 16 x 128 BF16, row stride D; rows >= nvalid are ignored.  m5/l5/acc5: the running partial [GMAX], [GMAX], [GMAX][D].
+__device__ __forceinline__ void raw_rows_attend(RawScratch& R, const u16* __restrict__ krows, const u16* __restrict__ vrows, int nvalid,
+                                                float scale_log2e, int G, int tid, float* __restrict__ m5, float* __restrict__ l5,
+                                                float (*__restrict__ acc5)[D]) {
+  __syncthreads();               // qs is filled / the previous call is done with sc
   const int t = tid >> 4, c = tid & 15;
-  const long base = (long)ch * A.tcap * D;
   float kr[8];
   {
     u32x4 kv = {0u, 0u, 0u, 0u};
-    if (t < TL) kv = *reinterpret_cast<const u32x4*>(A.kt + base + (long)t * D + 8 * c);
+    if (t < nvalid) kv = *reinterpret_cast<const u32x4*>(krows + t * D + 8 * c);
 #pragma unroll
     for (int i = 0; i < 4; ++i) { kr[2 * i] = bf16_bits_to_float(kv[i] & 0xFFFFu); kr[2 * i + 1] = bf16_bits_to_float(kv[i] >> 16); }
   }
   for (int g = 0; g < G; ++g) {
     float d = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) d += qs[g][8 * c + i] * kr[i];
+    for (int i = 0; i < 8; ++i) d += R.qs[g][8 * c + i] * kr[i];
 #pragma unroll
     for (int o = 8; o > 0; o >>= 1) d += __shfl_xor(d, o, 16);
-    if (c == 0) sc[g][t] = t < TL ? d * A.scale_log2e : -INFINITY;
+    if (c == 0) R.sc[g][t] = t < nvalid ? d * scale_log2e : -INFINITY;
   }
   __syncthreads();
-  {   // thread (g = tid >> 4, token = tid & 15): softmax over the 16 lanes of the row
+  {   // thread (g = tid >> 4, token = tid & 15): softmax over the 16 lanes of the row, merged into the running partial
     const int g = tid >> 4, tk = tid & 15;
-    float s = g < G ? sc[g][tk] : -INFINITY, m = s;
+    const float s = g < G ? R.sc[g][tk] : -INFINITY;
+    float mt = s;
 #pragma unroll
-    for (int o = 8; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 16));
-    const float mu = m == -INFINITY ? 0.f : m;
+    for (int o = 8; o > 0; o >>= 1) mt = fmaxf(mt, __shfl_xor(mt, o, 16));
+    const float m_old = g < G ? m5[g] : -INFINITY, m_new = fmaxf(m_old, mt), mu = m_new == -INFINITY ? 0.f : m_new;
     const float p = __builtin_amdgcn_exp2f(s - mu);
-    float l = p;
+    float lt = p;
 #pragma unroll
-    for (int o = 8; o > 0; o >>= 1) l += __shfl_xor(l, o, 16);
+    for (int o = 8; o > 0; o >>= 1) lt += __shfl_xor(lt, o, 16);
     __syncthreads();
     if (g < G) {
-      sc[g][tk] = p;
-      if (tk == 0) { const long pidx = (qh0 + g) * A.nslot + (A.nslot - 1); store_partial(A.pm + pidx, m); store_partial(A.pl + pidx, l); }
+      R.sc[g][tk] = p;
+      if (tk == 0) {
+        const float al = m_old == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_old - mu);
+        R.alpha[g] = al; m5[g] = m_new; l5[g] = l5[g] * al + lt;
+      }
     }
   }
   __syncthreads();
   const int d = tid & 127;
   for (int g = tid >> 7; g < G; g += 2) {
-    float acc = 0.f;
-    for (int tk = 0; tk < TL; ++tk) acc += sc[g][tk] * bf16_bits_to_float(A.vt[base + (long)tk * D + d]);
-    store_partial(A.pa + ((qh0 + g) * A.nslot + (A.nslot - 1)) * D + d, acc);
+    float acc = acc5[g][d] * R.alpha[g];
+    for (int tk = 0; tk < nvalid; ++tk) acc += R.sc[g][tk] * bf16_bits_to_float(vrows[tk * D + d]);
+    acc5[g][d] = acc;
   }
-  publish_and_merge(A, b * A.n_kv + kvh, qh0, G, tid);
 }
 
 // ---------------------------------------------------------------------------------------------------- block tables (LDS)
@@ -188,9 +199,10 @@ struct AttnLds {
   u32 sel[256];
   u32x4 bwk[2][NG], bwv[2][NG];
   u32x4 qw[GMAX][NG];
-  float m[4][GMAX], l[4][GMAX];
-  float acc[4][GMAX][D];
+  float m[5][GMAX], l[5][GMAX];   // per-wave partials of the block merge; [4] = the uncompressed rows
+  float acc[5][GMAX][D];          // acc[0..3] double as RawScratch before the waves publish and as the merge factors afterwards
 };
+static_assert(sizeof(RawScratch) <= 4 * GMAX * D * sizeof(float) && 4 * MAX_SLOTS <= 4 * GMAX * D, "scratch views must fit acc[0..3]");
 struct TableRegs { u32 b0, b1; u32 qlo[4], qhi[4]; };      // one thread's raw inputs of the per-block tables
 // global loads only (issued before the first tile's loads so that the two latencies overlap)
 __device__ __forceinline__ void tables_load(TableRegs& Tr, int tid, const AttnArgs& A, int brow, long qh0) {
@@ -418,17 +430,19 @@ __device__ __forceinline__ void consume(const TileRegs& R, WaveState& st, const 
 // ---------------------------------------------------------------------------------------------------- main kernel
 __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
   __shared__ AttnLds L;
-  const int bh = blockIdx.x, split = blockIdx.y, tid = threadIdx.x;
+  const int bh = blockIdx.x, tid = threadIdx.x;
+  // with a raw tail the grid has one more block row: it is dispatched first (blockIdx.y == 0), owns no compressed tile and writes
+  // partial slot nsplit
+  const int split = A.nslot > A.nsplit ? (blockIdx.y == 0 ? A.nsplit : (int)blockIdx.y - 1) : (int)blockIdx.y;
   const int b = bh / A.n_kv, kvh = bh % A.n_kv, G = A.G;
   const int slot = A.slot[b], ch = (slot < 0 ? 0 : slot) * A.n_kv + kvh;
-  if (split == A.nsplit) { tail_block(A, b, kvh, ch, slot); return; }
   const long qh0 = (long)b * A.n_q + (long)kvh * G;
   TableRegs Tr;
   tables_load(Tr, tid, A, ch % A.NB, qh0);
 
   const int S = slot < 0 ? 0 : A.sl[ch];
   const int ntiles = (S + T - 1) / T, chunk = (ntiles + A.nsplit - 1) / A.nsplit;
-  const int tlo = split * chunk, thi = min(tlo + chunk, ntiles);
+  const int tlo = min(split * chunk, ntiles), thi = min(tlo + chunk, ntiles);
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, a = lane & 15, q = lane >> 4;
   const long rowb = (long)ch * A.S_pad, tileb = (long)ch * (A.S_pad / T);
   Bases B;
@@ -452,6 +466,7 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
     load_tags(B, min(t0 + 4, tlast), a, Tg);
   }
   tables_store(L, Tr, tid);
+  if (tid < GMAX) { L.m[4][tid] = -INFINITY; L.l[4][tid] = 0.f; }
   __syncthreads();        // block tables are ready
   // Q as the B operand of the score product: lane (head a, quad q), product u covers group 4q+u in word order (e, e+4);
   // exponent-base words of the lane's units
@@ -494,6 +509,15 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
     load_tile(B, t, lane, Tg, R0);
     consume<true>(R0, st, L, B, Tg.kto, Tg.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
   }
+  // ---- the raw tail of the cache head: the extra block row
+  if (split == A.nsplit) {
+    RawScratch& R = *reinterpret_cast<RawScratch*>(&L.acc[0][0][0]);
+    const int TL = slot < 0 ? 0 : min(A.tl[ch], A.tcap);
+    for (int g = tid >> 7; g < G; g += 2) L.acc[4][g][tid & 127] = 0.f;
+    raw_rows_begin(R, A, qh0, G, tid);
+    raw_rows_attend(R, A.kt + (long)ch * A.tcap * D, A.vt + (long)ch * A.tcap * D, TL, A.scale_log2e, G, tid, L.m[4], L.l[4], L.acc[4]);
+    __syncthreads();      // the scratch view is dead before the waves publish into the same memory
+  }
   // The accumulators are MFMA results: keep their first non-MFMA read a full MFMA latency away on every path.
   asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");
   float l_run = quad_rows_sum(st.l_run);
@@ -513,10 +537,10 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
   for (int g = tid >> 7; g < G; g += 2) {
     float M = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) M = fmaxf(M, L.m[w][g]);
+    for (int w = 0; w < 5; ++w) M = fmaxf(M, L.m[w][g]);
     float Lc = 0.f, Ac = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < 5; ++w) {
       const float f = L.m[w][g] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(L.m[w][g] - M);
       Lc += L.l[w][g] * f; Ac += L.acc[w][g][d] * f;
     }
@@ -524,7 +548,7 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
     if (d == 0) { store_partial(A.pm + pidx, M); store_partial(A.pl + pidx, Lc); }
     store_partial(A.pa + pidx * D + d, Ac);
   }
-  publish_and_merge(A, bh, qh0, G, tid);
+  publish_and_merge(A, bh, qh0, G, tid, &L.acc[0][0][0]);
 }
 
 // ---------------------------------------------------------------------------------------------------- split merge

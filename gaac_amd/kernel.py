@@ -24,6 +24,12 @@ def choose_nsplit(B: int, n_kv: int, S: int, target_ctas: int = 512, min_tok: in
     return min(max(1, target_ctas // (B * n_kv)), max(1, S // min_tok), cap)
 
 
+def nsplit_with_tail_row(nsplit: int, B: int, n_kv: int, resident: int = 512) -> int:
+    """The raw tail adds one block row to the launch: give up one split when that row would no longer be resident together with the
+    others (2 blocks on each of the 256 CUs), so that no block has to wait for a free CU."""
+    return nsplit - 1 if nsplit > 1 and B * n_kv * nsplit <= resident < B * n_kv * (nsplit + 1) else nsplit
+
+
 class AttnWorkspace:
     """Output + split partials of one launch shape (fp32 m, l [rows*NSLOT] and acc [rows*NSLOT*D]; rows = B*n_q)."""
     def __init__(self, rows: int, nslot: int, dtype, dev, with_out: bool = True):
