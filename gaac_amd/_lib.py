@@ -20,6 +20,11 @@ _SIGNATURES = {
     "gaac_attn_split": [P] * 16 + [P, P, c_int, c_int, c_int, P, c_int, c_float, c_int, c_int, P, P, P, c_int, P, P, P, P],
     "gaac_attn_combine": [P, P, P, P, c_int, c_int, P],
     "gaac_cache_append": [P, c_int, c_int, P, P, P, P, c_int, c_int, c_int] + [P] * 18 + [P, P],
+    "gaac_paged_store": [P, P, c_long, c_long, P, c_int, P, c_int, P, P, P, P, P, P, P, P, P, P, c_int, P],
+    "gaac_paged_free": [P, c_int, P, P, P],
+    "gaac_paged_release": [P, c_int, P, P, P, c_int, P],
+    "gaac_paged_decode": [P, c_int, P, P, P, c_int, P, P, c_long, P, P, P, P, c_int, P],
+    "gaac_paged_attn": [P, c_int, P, P, P, c_int, P, c_int, P, c_int, c_int, c_int, c_float, c_int, P, P, P, P, c_int, P, P, P, P, P, P],
     "gaac_stream_copy": [P, P, c_long, P],
     "gaac_attn_fused": [P] * 16 + [P, P, c_int, c_int, c_int, P, c_int, c_float, c_int, c_int, P, P, P, c_int, P, P, P, P, P, P],
     "gaac_attn_launch": [P] * 16 + [P, P, c_int, c_int, c_int, P, c_int, c_float, c_int, c_int, P, P, P, c_int, P, P, P, P, P],

@@ -9,7 +9,7 @@ import os, subprocess, sys, shutil
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libgaac_hip.so")
-SOURCES = ["codec.hip", "attn.hip", "cache.hip"]
+SOURCES = ["codec.hip", "attn.hip", "cache.hip", "paged.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", 
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",      # never emit packed-FP32 VALU ops
          "-Wno-unused-command-line-argument"]

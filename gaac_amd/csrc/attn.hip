@@ -31,7 +31,12 @@ struct AttnArgs {
   int S_pad; float scale_log2e; int nsplit; int nslot; int n_kv; int n_q; int G; int NB;
   const u16* kt; const u16* vt; const int* tl; int tcap;
   int* tickets; u16* out;      // fused merge: one arrival counter per (batch row, kv head), zero between launches
+  // paged slot pool (k_attn_split<true>): sl = tokens per batch row, bt = block table [B][bt_stride], mt = mode table, pool = tile
+  // slots of TS bytes, raw = side pool of BF16 tiles; physical tile = block*2*n_kv + 2*kvh + kind
+  const uint8_t* pool; const u16* raw; const int* mt; const int* bt; int bt_stride; int TS;
 };
+constexpr int MAX_CHUNK = 1024;  // tiles per split whose slot lookups a block keeps in LDS (paged mode)
+constexpr int SLOT_CD = TILE_SM, SLOT_FL = TILE_SM + TILE_CD, SLOT_OV = SLOT_FL + 4 * T;      // byte offsets inside a tile slot
 
 __device__ __forceinline__ float bf16_bits_to_float(u32 h) { return __uint_as_float(h << 16); }
 __device__ __forceinline__ u32 pack_bf16x2(float lo, float hi) {
@@ -133,6 +138,7 @@ struct RawScratch {              // lives in the block-merge buffer, which is id
   float qs[GMAX][D];             // the query heads in fp32, natural channel order
   float sc[GMAX][T];             // scores, then probabilities
   float alpha[GMAX];             // rescale factor of the running partial
+  u16 krows[T * D], vrows[T * D];   // a compressed tile decoded next to a raw one (paged mode: only one kind of a tile is raw)
 };
 __device__ __forceinline__ void raw_rows_begin(RawScratch& R, const AttnArgs& A, long qh0, int G, int tid) {
   for (int i = tid; i < G * D; i += 256) R.qs[i >> 7][i & 127] = bf16_bits_to_float(A.q[qh0 * D + i]);
@@ -259,31 +265,58 @@ struct KindRegs {                // one lane's view of one tile (K or V)
   u32x2 e;                       // the 8 escape bytes from pos0 on
 };
 struct TileRegs { KindRegs k, v; };
-struct TagRegs { u32 kfl, vfl; u32 kto, vto; };
+struct TagRegs { u32 kfl, vfl; u32 kto, vto; int raw; };      // kto/vto: tile offset in the head's escape stream | slot index (paged)
 
-struct Bases {                   // uniform (scalar) views of one cache head
+struct Bases {                   // uniform (scalar) views of one cache head; paged mode uses kov = vov = pool and TS only
   const uint8_t* ksm; const uint8_t* kcd; const int* kfl; const int* kto; const uint8_t* kov;
   const uint8_t* vsm; const uint8_t* vcd; const int* vfl; const int* vto; const uint8_t* vov;
+  int TS;
 };
+struct TileTable { const int2* tt; int tlo; };      // paged mode: mode-table entries (K, V) of the block's tiles, in LDS
 
-__device__ __forceinline__ void load_tags(const Bases& B, int tile, int a, TagRegs& Tg) {
-  const unsigned w = (unsigned)(tile * T + a);
-  Tg.kfl = (u32)B.kfl[w]; Tg.vfl = (u32)B.vfl[w];
-  Tg.kto = (u32)B.kto[tile]; Tg.vto = (u32)B.vto[tile];
+// start of a tile's escape bytes
+template <bool PAGED>
+__device__ __forceinline__ const uint8_t* esc_of_tile(const uint8_t* ov, u32 to, int TS) {
+  return PAGED ? ov + (size_t)to * (size_t)TS + SLOT_OV : ov + to;
 }
 
+template <bool PAGED>
+__device__ __forceinline__ void load_tags(const Bases& B, const TileTable& TT, int tile, int a, TagRegs& Tg) {
+  if (PAGED) {
+    const int2 e = TT.tt[tile - TT.tlo];
+    const int ek = __builtin_amdgcn_readfirstlane(e.x), ev = __builtin_amdgcn_readfirstlane(e.y);
+    Tg.raw = (ek | ev) < 0;                       // a tile with a raw side is skipped here and handled by raw_rows_attend
+    Tg.kto = (u32)max(ek, 0); Tg.vto = (u32)max(ev, 0);
+    Tg.kfl = reinterpret_cast<const u32*>(B.kov + (size_t)Tg.kto * (size_t)B.TS + SLOT_FL)[a];
+    Tg.vfl = reinterpret_cast<const u32*>(B.vov + (size_t)Tg.vto * (size_t)B.TS + SLOT_FL)[a];
+  } else {
+    const unsigned w = (unsigned)(tile * T + a);
+    Tg.kfl = (u32)B.kfl[w]; Tg.vfl = (u32)B.vfl[w];
+    Tg.kto = (u32)B.kto[tile]; Tg.vto = (u32)B.vto[tile];
+    Tg.raw = 0;
+  }
+}
+
+template <bool PAGED>
 __device__ __forceinline__ void load_tile(const Bases& B, int tile, int lane, const TagRegs& Tg, TileRegs& R) {
   const int q = lane >> 4;
-  load_payload(B.ksm + (size_t)tile * TILE_SM, B.kcd + (size_t)tile * TILE_CD, lane, R.k.pay);
-  load_payload(B.vsm + (size_t)tile * TILE_SM, B.vcd + (size_t)tile * TILE_CD, lane, R.v.pay);
+  if (PAGED) {
+    const uint8_t* ks = B.kov + (size_t)__builtin_amdgcn_readfirstlane(Tg.kto) * (size_t)B.TS;
+    const uint8_t* vs = B.vov + (size_t)__builtin_amdgcn_readfirstlane(Tg.vto) * (size_t)B.TS;
+    load_payload(ks, ks + SLOT_CD, lane, R.k.pay);
+    load_payload(vs, vs + SLOT_CD, lane, R.v.pay);
+  } else {
+    load_payload(B.ksm + (size_t)tile * TILE_SM, B.kcd + (size_t)tile * TILE_CD, lane, R.k.pay);
+    load_payload(B.vsm + (size_t)tile * TILE_SM, B.vcd + (size_t)tile * TILE_CD, lane, R.v.pay);
+  }
   // escape bytes per line of K (low half) and V (high half): one scan for both
   const u32 rb = (u32)esc_bytes(Tg.kfl) | ((u32)esc_bytes(Tg.vfl) << 16);
   const u32 excl = row_scan16(rb) - rb;
   R.k.f = Tg.kfl; R.v.f = Tg.vfl;
   R.k.pos0 = (excl & 0xFFFFu) + (u32)esc_prefix(Tg.kfl, 8 * q);
   R.v.pos0 = (excl >> 16) + (u32)esc_prefix(Tg.vfl, 8 * q);
-  R.k.e = load_u32x2_unaligned(B.kov + Tg.kto + R.k.pos0);
-  R.v.e = load_u32x2_unaligned(B.vov + Tg.vto + R.v.pos0);
+  R.k.e = load_u32x2_unaligned(esc_of_tile<PAGED>(B.kov, PAGED ? __builtin_amdgcn_readfirstlane(Tg.kto) : Tg.kto, B.TS) + R.k.pos0);
+  R.v.e = load_u32x2_unaligned(esc_of_tile<PAGED>(B.vov, PAGED ? __builtin_amdgcn_readfirstlane(Tg.vto) : Tg.vto, B.TS) + R.v.pos0);
 }
 
 // ---------------------------------------------------------------------------------------------------- one tile pair
@@ -352,15 +385,15 @@ __device__ __forceinline__ bool tier0(u32 tag8, int u) { return (tag8 & (1u << (
 
 // PARTIAL: the tile is the last one of the sequence and only partly filled (rows >= S are masked out).  It is a template
 // parameter, not a run-time branch, so that no branch separates the score MFMAs from the first read of their result.
-template <bool PARTIAL, bool SLOW>
+template <bool PAGED, bool PARTIAL, bool SLOW>
 __device__ __forceinline__ void consume_tile(const TileRegs& R, WaveState& st, const AttnLds& L, const Bases& B,
                                              u32 kto, u32 vto, int tile, int S, float scale_log2e, int a, int q,
                                              const u32x4 (&qf)[4], const u32x4 (&kb3)[4], const u32x4 (&kb4)[4],
                                              const u32x4& vb3, const u32x4& vb4) {
   u32 ktag8, vtag8;
   u32x4 xk[4], xv[4];
-  unit_x_words<KIND_K, SLOW>(R.k, L, B.kov + kto, q, kb4, ktag8, xk);
-  unit_x_words<KIND_V, SLOW>(R.v, L, B.vov + vto, q, &vb4, vtag8, xv);
+  unit_x_words<KIND_K, SLOW>(R.k, L, esc_of_tile<PAGED>(B.kov, kto, B.TS), q, kb4, ktag8, xk);
+  unit_x_words<KIND_V, SLOW>(R.v, L, esc_of_tile<PAGED>(B.vov, vto, B.TS), q, &vb4, vtag8, xv);
   // ---- scores: S[tok 4q+r][head a]
   f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -416,38 +449,53 @@ __device__ __forceinline__ void consume_tile(const TileRegs& R, WaveState& st, c
 }
 
 // A tile needs the SLOW instantiation when some lane holds two or more raw groups (about 1 tile in 100 at 0.3 % raw groups).
-template <bool PARTIAL>
+template <bool PAGED, bool PARTIAL>
 __device__ __forceinline__ void consume(const TileRegs& R, WaveState& st, const AttnLds& L, const Bases& B, u32 kto, u32 vto, int tile,
                                         int S, float scale_log2e, int a, int q, const u32x4 (&qf)[4], const u32x4 (&kb3)[4],
                                         const u32x4 (&kb4)[4], const u32x4& vb3, const u32x4& vb4) {
   const u32 kr = __builtin_amdgcn_ubfe(R.k.f, 8 * q, 8) & 0xAAu, vr = __builtin_amdgcn_ubfe(R.v.f, 8 * q, 8) & 0xAAu;
   if (__builtin_expect(__builtin_amdgcn_ballot_w64(((kr & (kr - 1u)) | (vr & (vr - 1u))) != 0u) != 0, 0))
-    consume_tile<PARTIAL, true>(R, st, L, B, kto, vto, tile, S, scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+    consume_tile<PAGED, PARTIAL, true>(R, st, L, B, kto, vto, tile, S, scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
   else
-    consume_tile<PARTIAL, false>(R, st, L, B, kto, vto, tile, S, scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+    consume_tile<PAGED, PARTIAL, false>(R, st, L, B, kto, vto, tile, S, scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
 }
 
 // ---------------------------------------------------------------------------------------------------- main kernel
+template <bool PAGED>
 __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
   __shared__ AttnLds L;
+  __shared__ int2 tile_table[PAGED ? MAX_CHUNK : 1];
   const int bh = blockIdx.x, tid = threadIdx.x;
   // with a raw tail the grid has one more block row: it is dispatched first (blockIdx.y == 0), owns no compressed tile and writes
   // partial slot nsplit
   const int split = A.nslot > A.nsplit ? (blockIdx.y == 0 ? A.nsplit : (int)blockIdx.y - 1) : (int)blockIdx.y;
   const int b = bh / A.n_kv, kvh = bh % A.n_kv, G = A.G;
-  const int slot = A.slot[b], ch = (slot < 0 ? 0 : slot) * A.n_kv + kvh;
+  const int slot = PAGED ? 0 : A.slot[b], ch = PAGED ? kvh : (slot < 0 ? 0 : slot) * A.n_kv + kvh;
   const long qh0 = (long)b * A.n_q + (long)kvh * G;
   TableRegs Tr;
   tables_load(Tr, tid, A, ch % A.NB, qh0);
 
-  const int S = slot < 0 ? 0 : A.sl[ch];
-  const int ntiles = (S + T - 1) / T, chunk = (ntiles + A.nsplit - 1) / A.nsplit;
+  const int S = PAGED ? max(A.sl[b], 0) : (slot < 0 ? 0 : A.sl[ch]);
+  const int ntiles = (S + T - 1) / T, chunk = PAGED ? min((ntiles + A.nsplit - 1) / A.nsplit, MAX_CHUNK) : (ntiles + A.nsplit - 1) / A.nsplit;
   const int tlo = min(split * chunk, ntiles), thi = min(tlo + chunk, ntiles);
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, a = lane & 15, q = lane >> 4;
-  const long rowb = (long)ch * A.S_pad, tileb = (long)ch * (A.S_pad / T);
   Bases B;
-  B.ksm = A.k.sm + rowb * D; B.kcd = A.k.cd + rowb * CB; B.kfl = A.k.flags + rowb; B.kto = A.k.tile_off + tileb; B.kov = A.k.ovf + A.k.head_start[ch];
-  B.vsm = A.v.sm + rowb * D; B.vcd = A.v.cd + rowb * CB; B.vfl = A.v.flags + rowb; B.vto = A.v.tile_off + tileb; B.vov = A.v.ovf + A.v.head_start[ch];
+  TileTable TT{tile_table, tlo};
+  if (PAGED) {
+    // logical tile -> block table -> mode table (paged_kernel.py:137-138), resolved once per block into LDS
+    B.kov = B.vov = A.pool; B.TS = A.TS;
+    B.ksm = B.kcd = B.vsm = B.vcd = nullptr; B.kfl = B.kto = B.vfl = B.vto = nullptr;
+    for (int i = tid; i < thi - tlo; i += 256) {
+      const long pc = (long)A.bt[(long)b * A.bt_stride + tlo + i] * (2 * A.n_kv) + 2 * kvh;
+      tile_table[i] = int2{A.mt[pc], A.mt[pc + 1]};
+    }
+    __syncthreads();
+  } else {
+    const long rowb = (long)ch * A.S_pad, tileb = (long)ch * (A.S_pad / T);
+    B.ksm = A.k.sm + rowb * D; B.kcd = A.k.cd + rowb * CB; B.kfl = A.k.flags + rowb; B.kto = A.k.tile_off + tileb; B.kov = A.k.ovf + A.k.head_start[ch];
+    B.vsm = A.v.sm + rowb * D; B.vcd = A.v.cd + rowb * CB; B.vfl = A.v.flags + rowb; B.vto = A.v.tile_off + tileb; B.vov = A.v.ovf + A.v.head_start[ch];
+    B.TS = 0;
+  }
 
   // tiles of this wave: t(i) = tlo + wave + 4 i, i < n.  Ping-pong registers R0/R1; tag words are fetched one tile further
   // ahead (index clamped to the wave's last tile, so that no load sits under a branch the consumer has to join).  A partly
@@ -460,10 +508,10 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
   TileRegs R0, R1;
   TagRegs Tg, TgC0, TgC1;
   if (n > 0) {          // start the first tile's loads before waiting for the block tables
-    load_tags(B, t0, a, Tg);
+    load_tags<PAGED>(B, TT, t0, a, Tg);
     TgC0 = Tg;
-    load_tile(B, t0, lane, Tg, R0);
-    load_tags(B, min(t0 + 4, tlast), a, Tg);
+    load_tile<PAGED>(B, t0, lane, Tg, R0);
+    load_tags<PAGED>(B, TT, min(t0 + 4, tlast), a, Tg);
   }
   tables_store(L, Tr, tid);
   if (tid < GMAX) { L.m[4][tid] = -INFINITY; L.l[4][tid] = 0.f; }
@@ -485,32 +533,60 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
     for (; i + 2 < n; i += 2) {
       const int t = t0 + 4 * i;
       TgC1 = Tg;
-      load_tile(B, t + 4, lane, Tg, R1);
-      load_tags(B, min(t + 8, tlast), a, Tg);
-      consume<false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+      load_tile<PAGED>(B, t + 4, lane, Tg, R1);
+      load_tags<PAGED>(B, TT, min(t + 8, tlast), a, Tg);
+      if (!PAGED || !TgC0.raw) consume<PAGED, false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
       TgC0 = Tg;
-      load_tile(B, t + 8, lane, Tg, R0);
-      load_tags(B, min(t + 12, tlast), a, Tg);
-      consume<false>(R1, st, L, B, TgC1.kto, TgC1.vto, t + 4, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+      load_tile<PAGED>(B, t + 8, lane, Tg, R0);
+      load_tags<PAGED>(B, TT, min(t + 12, tlast), a, Tg);
+      if (!PAGED || !TgC1.raw) consume<PAGED, false>(R1, st, L, B, TgC1.kto, TgC1.vto, t + 4, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
     }
     const int t = t0 + 4 * i;
     if (n - i == 2) {
       TgC1 = Tg;
-      load_tile(B, t + 4, lane, Tg, R1);
-      consume<false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
-      consume<false>(R1, st, L, B, TgC1.kto, TgC1.vto, t + 4, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+      load_tile<PAGED>(B, t + 4, lane, Tg, R1);
+      if (!PAGED || !TgC0.raw) consume<PAGED, false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+      if (!PAGED || !TgC1.raw) consume<PAGED, false>(R1, st, L, B, TgC1.kto, TgC1.vto, t + 4, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
     } else {
-      consume<false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+      if (!PAGED || !TgC0.raw) consume<PAGED, false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
     }
   }
   if (own_partial) {
     const int t = ntiles - 1;
-    load_tags(B, t, a, Tg);
-    load_tile(B, t, lane, Tg, R0);
-    consume<true>(R0, st, L, B, Tg.kto, Tg.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+    load_tags<PAGED>(B, TT, t, a, Tg);
+    load_tile<PAGED>(B, t, lane, Tg, R0);
+    if (!PAGED || !Tg.raw) consume<PAGED, true>(R0, st, L, B, Tg.kto, Tg.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
   }
-  // ---- the raw tail of the cache head: the extra block row
-  if (split == A.nsplit) {
+  // ---- rows kept as plain BF16: the raw tail of a cache head (the extra block row) or, in the paged pool, tiles of this split
+  // whose K or V side is a raw tile (the block that is still filling, or escapes that did not fit the slot)
+  if (PAGED) {
+    bool mine = false;
+    for (int i = tid; i < thi - tlo; i += 256) mine |= (tile_table[i].x | tile_table[i].y) < 0;
+    if (__syncthreads_or(mine)) {
+      RawScratch& R = *reinterpret_cast<RawScratch*>(&L.acc[0][0][0]);
+      for (int g = tid >> 7; g < G; g += 2) L.acc[4][g][tid & 127] = 0.f;
+      raw_rows_begin(R, A, qh0, G, tid);
+      const uint8_t* b3k = A.k.base3 + (long)(ch % A.NB) * D; const uint8_t* b4k = A.k.base4 + (long)(ch % A.NB) * D;
+      const uint8_t* b3v = A.v.base3 + (long)(ch % A.NB) * D; const uint8_t* b4v = A.v.base4 + (long)(ch % A.NB) * D;
+      for (int i = 0; i < thi - tlo; ++i) {
+        const int2 e = tile_table[i];
+        if ((e.x | e.y) >= 0) continue;
+        const u16* krows = R.krows; const u16* vrows = R.vrows;
+        if (e.x < 0) krows = A.raw + (long)(~e.x) * T * D;
+        else if (wave == 0) {
+          const uint8_t* sl = A.pool + (size_t)e.x * (size_t)A.TS;
+          decode_tile_rows<KIND_K>(sl, sl + SLOT_CD, reinterpret_cast<const int*>(sl + SLOT_FL), sl + SLOT_OV, b3k, b4k, lane, T, R.krows, D);
+        }
+        if (e.y < 0) vrows = A.raw + (long)(~e.y) * T * D;
+        else if (wave == 1) {
+          const uint8_t* sl = A.pool + (size_t)e.y * (size_t)A.TS;
+          decode_tile_rows<KIND_V>(sl, sl + SLOT_CD, reinterpret_cast<const int*>(sl + SLOT_FL), sl + SLOT_OV, b3v, b4v, lane, T, R.vrows, D);
+        }
+        raw_rows_attend(R, krows, vrows, min(T, S - (tlo + i) * T), A.scale_log2e, G, tid, L.m[4], L.l[4], L.acc[4]);
+        __syncthreads();      // staging rows are free again
+      }
+    }
+  } else if (split == A.nsplit) {
     RawScratch& R = *reinterpret_cast<RawScratch*>(&L.acc[0][0][0]);
     const int TL = slot < 0 ? 0 : min(A.tl[ch], A.tcap);
     for (int g = tid >> 7; g < G; g += 2) L.acc[4][g][tid & 127] = 0.f;
@@ -541,8 +617,9 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
     float Lc = 0.f, Ac = 0.f;
 #pragma unroll
     for (int w = 0; w < 5; ++w) {
-      const float f = L.m[w][g] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(L.m[w][g] - M);
-      Lc += L.l[w][g] * f; Ac += L.acc[w][g][d] * f;
+      const bool live = L.m[w][g] != -INFINITY;          // an empty partial's accumulator may hold anything
+      const float f = live ? __builtin_amdgcn_exp2f(L.m[w][g] - M) : 0.f;
+      Lc += L.l[w][g] * f; Ac += live ? L.acc[w][g][d] * f : 0.f;
     }
     const long pidx = (qh0 + g) * A.nslot + split;
     if (d == 0) { store_partial(A.pm + pidx, M); store_partial(A.pl + pidx, Lc); }
@@ -620,7 +697,8 @@ static int attn_split_impl(
   A.kt = (const u16*)kt; A.vt = (const u16*)vt; A.tl = TL; A.tcap = TCAP;
   A.tickets = tickets; A.out = (u16*)out;
   GAAC_REQUIRE(!tickets || out, "gaac_attn: the fused merge needs an output buffer");
-  hipLaunchKernelGGL(k_attn_split, dim3(B * n_kv, nslot), dim3(256), 0, (hipStream_t)stream, A);
+  A.pool = nullptr; A.raw = nullptr; A.mt = nullptr; A.bt = nullptr; A.bt_stride = 0; A.TS = 0;
+  hipLaunchKernelGGL(k_attn_split<false>, dim3(B * n_kv, nslot), dim3(256), 0, (hipStream_t)stream, A);
   return launch_status("gaac_attn(split)");
 }
 
@@ -661,4 +739,29 @@ extern "C" int gaac_attn_fused(
   GAAC_REQUIRE(out && tickets, "gaac_attn_fused: null output or ticket buffer");
   return attn_split_impl(smk, ck, fk, tok, ovk, ohsk, b3k, b4k, smv, cv, fv, tov, ovv, ohsv, b3v, b4v, q, slot, B, n_q, n_kv, SL, S_pad,
                          scale, nsplit, NB, kt, vt, TL, TCAP, pm, pl, pa, tickets, out, stream);
+}
+
+extern "C" int gaac_paged_attn(
+    const uint8_t* pool, int TS, const void* raw, const int* mt, const int* bt, int bt_stride, const int* seq_lens, int max_seq_len,
+    const void* q, int B, int n_q, int n_kv, float scale, int nsplit,
+    const uint8_t* b3k, const uint8_t* b4k, const uint8_t* b3v, const uint8_t* b4v, int NB,
+    float* pm, float* pl, float* pa, int* tickets, void* out, void* stream) {
+  GAAC_REQUIRE(n_kv > 0 && n_q > 0 && n_q % n_kv == 0 && n_q / n_kv <= GMAX, "GQA group size must be 1..%d (n_q=%d, n_kv=%d)", GMAX, n_q, n_kv);
+  GAAC_REQUIRE(pool && raw && mt && bt && seq_lens && q && b3k && b4k && b3v && b4v && pm && pl && pa && tickets && out, "gaac_paged_attn: null pointer");
+  GAAC_REQUIRE(B > 0 && NB > 0 && TS >= SLOT_OV && TS % 16 == 0 && bt_stride > 0, "gaac_paged_attn: bad sizes B=%d NB=%d TS=%d", B, NB, TS);
+  GAAC_REQUIRE(nsplit >= 1 && nsplit <= MAX_SLOTS, "gaac_paged_attn: nsplit must be in 1..%d", MAX_SLOTS);
+  const long max_tiles = ((long)max_seq_len + T - 1) / T;
+  GAAC_REQUIRE(max_seq_len >= 0 && max_tiles <= (long)bt_stride && (max_tiles + nsplit - 1) / nsplit <= MAX_CHUNK,
+               "gaac_paged_attn: max_seq_len %d needs at most %d blocks per row and at least %ld splits", max_seq_len, bt_stride, (max_tiles + MAX_CHUNK - 1) / MAX_CHUNK);
+  AttnArgs A;
+  A.k = StoreView{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, b3k, b4k};
+  A.v = StoreView{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, b3v, b4v};
+  A.q = (const u16*)q; A.pm = pm; A.pl = pl; A.pa = pa; A.slot = nullptr; A.sl = seq_lens;
+  A.S_pad = 0; A.scale_log2e = scale * 1.4426950408889634f; A.nsplit = nsplit; A.nslot = nsplit;
+  A.n_kv = n_kv; A.n_q = n_q; A.G = n_q / n_kv; A.NB = NB;
+  A.kt = nullptr; A.vt = nullptr; A.tl = nullptr; A.tcap = 0;
+  A.tickets = tickets; A.out = (u16*)out;
+  A.pool = pool; A.raw = (const u16*)raw; A.mt = mt; A.bt = bt; A.bt_stride = bt_stride; A.TS = TS;
+  hipLaunchKernelGGL(k_attn_split<true>, dim3(B * n_kv, nsplit), dim3(256), 0, (hipStream_t)stream, A);
+  return launch_status("gaac_paged_attn");
 }

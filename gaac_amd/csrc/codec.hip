@@ -111,34 +111,13 @@ __global__ void __launch_bounds__(64) k_decode_tiles(const uint8_t* __restrict__
                                                      const int* __restrict__ head_start, const uint8_t* __restrict__ base3,
                                                      const uint8_t* __restrict__ base4, int n_kv, const int* __restrict__ bidx,
                                                      int S, int S_pad, u16* __restrict__ out, long out_head_stride, long out_row_stride) {
-  const int tile = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, a = lane & 15, q = lane >> 4;
+  const int tile = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int brow = bidx ? bidx[h] : h % n_kv;
   const long row0 = (long)h * S_pad + (long)tile * T;
-  Payload P;
-  load_payload(sm + row0 * D, cd + row0 * CB, lane, P);
-  const u32 tag_word = (u32)flags[row0 + a];      // rows beyond S carry tag 0 (the encoder writes every word of a tile)
-  UnitMeta M;
-  tile_unit_meta(tag_word, lane, M);
-  const uint8_t* esc = ovf + head_start[h] + tile_off[(long)h * (S_pad / T) + tile];
-  u32 b3w[4], b4w[4];
-  if (KIND == KIND_V) { load_base_words<KIND>(base3 + (long)brow * D, a, b3w); load_base_words<KIND>(base4 + (long)brow * D, a, b4w); }
-#pragma unroll
-  for (int u = 0; u < 4; ++u) {
-    const int tok = unit_token<KIND>(a, q, u), grp = unit_group<KIND>(a, q, u);
-    if (KIND == KIND_K) { load_base_words<KIND>(base3 + (long)brow * D, grp, b3w); load_base_words<KIND>(base4 + (long)brow * D, grp, b4w); }
-    u32 slo, shi, w[4];
-    unit_sm(P, u, slo, shi);
-    const u32 eb = M.tag[u] == 1u ? (u32)esc[M.pos[u]] : 0u;
-    decode_unit(slo, shi, unit_code_word(P.c0, P.c1, P.c2, u), M.tag[u], eb, esc + M.pos[u], b3w, b4w, w);
-    if (tile * T + tok < S) {
-      u16* o = out + (long)h * out_head_stride + (long)(tile * T + tok) * out_row_stride;
-#pragma unroll
-      for (int p = 0; p < 4; ++p) {
-        o[chan_of<KIND>(8 * grp + p)] = (u16)(w[p] & 0xFFFFu);
-        o[chan_of<KIND>(8 * grp + p + 4)] = (u16)(w[p] >> 16);
-      }
-    }
-  }
+  // rows beyond S carry tag 0 (the encoder writes every word of a tile) and are not written
+  decode_tile_rows<KIND>(sm + row0 * D, cd + row0 * CB, flags + row0, ovf + head_start[h] + tile_off[(long)h * (S_pad / T) + tile],
+                         base3 + (long)brow * D, base4 + (long)brow * D, lane, min(T, S - tile * T),
+                         out + (long)h * out_head_stride + (long)tile * T * out_row_stride, out_row_stride);
 }
 
 // Plain streaming copy with the access shape of the attention kernel's payload loads (16 B per lane, 1 KiB per wave-wide

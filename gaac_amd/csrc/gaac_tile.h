@@ -114,4 +114,38 @@ __device__ __forceinline__ void tile_unit_meta(u32 tag_word, int lane, UnitMeta&
   for (int u = 0; u < 4; ++u) { M.tag[u] = (tag_word >> (8 * q + 2 * u)) & 3u; M.pos[u] = pos; pos += tag_size(M.tag[u]); }
 }
 
+// Decodes one stored tile (native order) into 16 rows of 128 BF16 in natural channel order: row `tok` at out + tok*row_stride,
+// rows >= nvalid are not written.  esc: the tile's escape bytes; b3row / b4row: the 128 base bytes of the head (channel order).
+// One wave; bit-exact inverse of encode_staged_tile (codec.py:186-218).
+template <int KIND>
+__device__ __forceinline__ void decode_tile_rows(const uint8_t* __restrict__ sm_tile, const uint8_t* __restrict__ cd_tile,
+                                                 const int* __restrict__ flags_tile, const uint8_t* __restrict__ esc,
+                                                 const uint8_t* __restrict__ b3row, const uint8_t* __restrict__ b4row, int lane, int nvalid,
+                                                 u16* __restrict__ out, long row_stride) {
+  const int a = lane & 15, q = lane >> 4;
+  Payload P;
+  load_payload(sm_tile, cd_tile, lane, P);
+  UnitMeta M;
+  tile_unit_meta((u32)flags_tile[a], lane, M);
+  u32 b3w[4], b4w[4];
+  if (KIND == KIND_V) { load_base_words<KIND>(b3row, a, b3w); load_base_words<KIND>(b4row, a, b4w); }
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int tok = unit_token<KIND>(a, q, u), grp = unit_group<KIND>(a, q, u);
+    if (KIND == KIND_K) { load_base_words<KIND>(b3row, grp, b3w); load_base_words<KIND>(b4row, grp, b4w); }
+    u32 slo, shi, w[4];
+    unit_sm(P, u, slo, shi);
+    const u32 eb = M.tag[u] == 1u ? (u32)esc[M.pos[u]] : 0u;
+    decode_unit(slo, shi, unit_code_word(P.c0, P.c1, P.c2, u), M.tag[u], eb, esc + M.pos[u], b3w, b4w, w);
+    if (tok < nvalid) {
+      u16* o = out + (long)tok * row_stride;
+#pragma unroll
+      for (int p = 0; p < 4; ++p) {
+        o[chan_of<KIND>(8 * grp + p)] = (u16)(w[p] & 0xFFFFu);
+        o[chan_of<KIND>(8 * grp + p + 4)] = (u16)(w[p] >> 16);
+      }
+    }
+  }
+}
+
 }  // namespace gaac

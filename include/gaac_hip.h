@@ -96,6 +96,34 @@ int gaac_cache_append(
     void* v_tail, const uint8_t* v_base3, const uint8_t* v_base4, uint8_t* v_sm, uint8_t* v_codes, int* v_flags, uint8_t* v_ovf, int* v_tile_off, int* v_ovf_used,
     int* err, void* stream);
 
+/* ---- paged slot pool (the layout of /root/reference/gaac/vllm/paged_kernel.py:3-6 and store.py:17-19) -------------------------------
+ * pool: tile slots of TS bytes, physical tile p = block*2*n_kv + 2*kvh + kind: [0,2048) sign/mantissa | [2048,2816) codes |
+ * [2816,2880) 16 tag words | [2880,TS) escape bytes.  mt int32 [num_blocks*2*n_kv]: p = compressed in its slot, ~r = raw BF16 tile r of
+ * raw [tiles][16][128].  stack/top: free raw tiles; err: failed pops.  Bases uint8 [n_kv,128]. */
+
+/* LayerState.store -> _store_tiles, store.py:22-105.  key/value: bf16 rows [num_tokens][n_kv][128] with row strides in elements;
+ * ent int32 [n_ent][4] = (block, first token row, offset in block, rows), block < 0 = inactive; freeq int32 [n_ent*2*n_kv] receives
+ * the raw tiles to give back (-1 = none); call gaac_paged_free on it afterwards (pops and pushes never share a launch). */
+int gaac_paged_store(const void* key, const void* value, long k_stride, long v_stride, const int* ent, int n_ent,
+                     uint8_t* pool, int TS, void* raw, int* mt, int* stack, int* top, int* err, int* freeq,
+                     const uint8_t* b3k, const uint8_t* b4k, const uint8_t* b3v, const uint8_t* b4v, int n_kv, void* stream);
+/* _free_tiles, store.py:108-114. */
+int gaac_paged_free(const int* freeq, int n_items, int* stack, int* top, void* stream);
+/* LayerState.release_blocks -> _release_blocks, store.py:164-174: raw tiles of dead blocks go back, their mode entries are reset. */
+int gaac_paged_release(const int* blocks, int n_blocks, int* mt, int* stack, int* top, int n_kv, void* stream);
+/* LayerState.decode_blocks -> _decode_tiles, store.py:117-161: pairs int32 [n_pairs][3] = (block, first output row, valid rows <= 16);
+ * sk/sv: bf16 [rows][n_kv][128] with row stride row_stride elements. */
+int gaac_paged_decode(const uint8_t* pool, int TS, const void* raw, const int* mt, const int* pairs, int n_pairs, void* sk, void* sv,
+                      long row_stride, const uint8_t* b3k, const uint8_t* b4k, const uint8_t* b3v, const uint8_t* b4v, int n_kv, void* stream);
+/* paged_attention -> gaac_vpaged_launch, paged_kernel.py:42-277: decode attention of B rows over the pool through the block table
+ * bt int32 [B][bt_stride] and the mode table; seq_lens int32 [B] (tokens incl. the filling block; no separate tail); max_seq_len =
+ * an upper bound of seq_lens known to the host (bounds the tiles per split, at most 1024).  Partials pm, pl [B*n_q*nsplit],
+ * pa [B*n_q*nsplit*128], tickets int32 [B*n_kv] (zero) as in gaac_attn_fused; out bf16 [B*n_q][128]. */
+int gaac_paged_attn(const uint8_t* pool, int TS, const void* raw, const int* mt, const int* bt, int bt_stride, const int* seq_lens,
+                    int max_seq_len, const void* q, int B, int n_q, int n_kv, float scale, int nsplit,
+                    const uint8_t* b3k, const uint8_t* b4k, const uint8_t* b3v, const uint8_t* b4v, int NB,
+                    float* pm, float* pl, float* pa, int* tickets, void* out, void* stream);
+
 /* Measurement aid with no counterpart in the reference: a plain copy of nbytes (multiple of 16) with 16-byte accesses per lane,
  * the known-size kernel that HBM traffic counters (FETCH_SIZE / WRITE_SIZE) are scaled against. */
 int gaac_stream_copy(const void* src, void* dst, long nbytes, void* stream);

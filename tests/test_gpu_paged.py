@@ -1,0 +1,158 @@
+"""GPU tests of the paged slot pool: store path (filling blocks stay raw, full blocks are compressed in their slot or stay raw when
+their escapes do not fit), block decode (bit-exact) and decode attention through a permuted block table, against the history
+kept on the host and the oracle's fp32 attention.  Tolerance of /root/reference/tests/test_kernel.py:19."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gaac_oracle as O
+from common import kv_like16, to_bf16, to_u16, randn_bf16
+from gpu_util import require_gpu
+
+pytestmark = pytest.mark.gpu
+N_KV, G = 4, 4
+SCALE = 128 ** -0.5
+
+
+def _tok16(x16):
+    return np.ascontiguousarray(x16.transpose(1, 0, 2))
+
+
+def _bases(dev, seed=30):
+    from gaac_amd.codec import exponent_hist, bases_from_hist
+    out = {}
+    for name, sd, ss in (("k", seed, 2000), ("v", seed + 1, 2001)):
+        x = to_bf16(_tok16(kv_like16(N_KV, 2048, seed=sd, scale_seed=ss)), dev)
+        out[name + "3"], out[name + "4"] = bases_from_hist(exponent_hist(x, N_KV), N_KV)
+    return out
+
+
+class _Pool:
+    """A little scheduler: block pool + permuted block table + per-sequence history on the host."""
+    def __init__(self, dev, n_seq, max_blocks, num_blocks, raw_tiles, ovf_slot=128, seed=0):
+        from gaac_amd.paged import LayerState
+        self.dev = dev
+        self.st = LayerState(num_blocks, N_KV, raw_tiles, _bases(dev), ovf_slot, dev)
+        self.buf = torch.zeros(LayerState.pool_bytes(num_blocks, N_KV, ovf_slot), dtype=torch.uint8, device=dev)
+        perm = np.random.default_rng(seed).permutation(num_blocks)[:n_seq * max_blocks].reshape(n_seq, max_blocks)
+        self.bt_cpu = perm.astype(np.int32)
+        self.bt = torch.from_numpy(self.bt_cpu).to(dev)
+        self.lens = [0] * n_seq
+        self.hist = [(np.zeros((0, N_KV, 128), np.uint16), np.zeros((0, N_KV, 128), np.uint16)) for _ in range(n_seq)]
+
+    def step(self, new):
+        """new: {seq: (k16 [n, n_kv, 128], v16)}; stores the rows and extends the history."""
+        from gaac_amd.paged import build_store_entries
+        seqs = sorted(new)
+        ent = build_store_entries([self.lens[s] for s in seqs], [len(new[s][0]) for s in seqs], [self.bt_cpu[s] for s in seqs])
+        k = to_bf16(np.concatenate([new[s][0] for s in seqs]), self.dev); v = to_bf16(np.concatenate([new[s][1] for s in seqs]), self.dev)
+        self.st.store(k, v, self.buf, torch.from_numpy(ent).to(self.dev))
+        for s in seqs:
+            self.hist[s] = (np.concatenate([self.hist[s][0], new[s][0]]), np.concatenate([self.hist[s][1], new[s][1]]))
+            self.lens[s] += len(new[s][0])
+
+    def check(self, seqs, q16, nsplit=None):
+        from gaac_amd.paged import choose_nsplit
+        sl = torch.tensor([self.lens[s] for s in seqs], dtype=torch.int32, device=self.dev)
+        bt = self.bt[torch.tensor(seqs, device=self.dev)].contiguous()
+        ns = nsplit or choose_nsplit(len(seqs), N_KV, max(self.lens))
+        out = self.st.attention(to_bf16(q16, self.dev), self.buf, bt, sl, ns, max_seq_len=max(max(self.lens), 1))
+        got = O.bf16_to_f32(to_u16(out)).reshape(len(seqs), N_KV * G, 128)
+        for b, s in enumerate(seqs):
+            if self.lens[s] == 0:
+                assert np.abs(got[b]).max() == 0
+                continue
+            ref = O.ref_attention(q16[b], self.hist[s][0], self.hist[s][1], SCALE)
+            assert np.abs(got[b] - ref).max() <= 2e-2 * np.abs(ref).max() + 1e-3, (s, self.lens[s])
+        self.check_decode(seqs)
+
+    def check_decode(self, seqs):
+        pairs, row = [], 0
+        for s in seqs:
+            for lb in range(-(-self.lens[s] // 16)):
+                nv = min(16, self.lens[s] - 16 * lb)
+                pairs.append((int(self.bt_cpu[s][lb]), row, nv)); row += nv
+        if not pairs: return
+        sk = torch.zeros(row, N_KV, 128, dtype=torch.bfloat16, device=self.dev); sv = torch.zeros_like(sk)
+        self.st.decode_blocks(self.buf, torch.tensor(pairs, dtype=torch.int32, device=self.dev), sk, sv)
+        wk = np.concatenate([self.hist[s][0] for s in seqs]); wv = np.concatenate([self.hist[s][1] for s in seqs])
+        assert np.array_equal(to_u16(sk), wk) and np.array_equal(to_u16(sv), wv)
+
+
+def _rows(n, seed):
+    return _tok16(kv_like16(N_KV, n, seed=seed, scale_seed=2000)), _tok16(kv_like16(N_KV, n, seed=seed + 500, scale_seed=2001))
+
+
+def test_prefill_then_decode_steps_through_a_permuted_block_table():
+    dev = require_gpu()
+    P = _Pool(dev, n_seq=4, max_blocks=40, num_blocks=200, raw_tiles=64)
+    P.step({0: _rows(37, 1), 1: _rows(500, 2), 3: _rows(16, 3)})          # prompts (sequence 2 stays empty for now)
+    P.check([1, 0, 3, 2], randn_bf16((4, N_KV * G, 128), seed=9, scale=0.1))
+    compressed = int((P.st.mt >= 0).sum()); total = P.st.mt.numel()
+    # sequences 0, 1 have one filling block each (2*n_kv raw tiles per block); every full block is compressed in place
+    assert total - compressed == 2 * 2 * N_KV and int(P.st.top) == 64 - 2 * 2 * N_KV
+    for step in range(36):
+        live = [0, 1, 3] if step % 3 else [1, 3, 2]
+        P.step({s: _rows(1, 1000 + 7 * step + s) for s in live})
+        if step % 11 == 0 or step == 35:
+            P.check([3, 2, 0, 1], randn_bf16((4, N_KV * G, 128), seed=200 + step, scale=0.1))
+    P.st.check()
+    # pops and pushes balance: the tiles off the stack are exactly the raw entries of the mode table, at least the filling blocks
+    filling = sum(1 for L in P.lens if L % 16)
+    n_raw = int((P.st.mt < 0).sum())
+    assert int(P.st.top) == 64 - n_raw and n_raw >= filling * 2 * N_KV
+    P.check([0, 1, 2, 3], randn_bf16((4, N_KV * G, 128), seed=77, scale=0.1), nsplit=1)
+    P.check([0, 1, 2, 3], randn_bf16((4, N_KV * G, 128), seed=78, scale=0.1), nsplit=7)
+
+
+def test_tiles_whose_escapes_do_not_fit_stay_raw_and_blocks_are_released():
+    dev = require_gpu()
+    P = _Pool(dev, n_seq=2, max_blocks=8, num_blocks=32, raw_tiles=72, ovf_slot=32)
+    # sequence 0: ordinary rows (about 30 escape bytes per tile: some tiles fit the 32-byte slot, some do not);
+    # sequence 1: exponents far from every base -> every group raw (1280 escape bytes per tile)
+    rng = np.random.default_rng(3)
+    k_far = (rng.integers(0, 2, (48, N_KV, 128)) << 15 | 95 << 7 | rng.integers(0, 128, (48, N_KV, 128))).astype(np.uint16)      # ~2^-32
+    v_far = (rng.integers(0, 2, (48, N_KV, 128)) << 15 | 150 << 7 | rng.integers(0, 128, (48, N_KV, 128))).astype(np.uint16)     # ~2^23
+    P.step({0: _rows(64, 5), 1: (k_far, v_far)})
+    P.st.check()
+    n_raw = int((P.st.mt < 0).sum())
+    assert n_raw >= 3 * 2 * N_KV                                 # at least all of sequence 1
+    assert int(P.st.top) == 72 - n_raw
+    P.check([0, 1], randn_bf16((2, N_KV * G, 128), seed=5, scale=0.2), nsplit=2)
+    # a mixed tile (K compressed, V raw or the other way round) must have occurred for the check above to cover that path
+    mt = P.st.mt.cpu().numpy().reshape(-1, N_KV, 2)
+    used = np.unique(P.bt_cpu[0][:4])
+    mixed = sum(int((mt[b, h, 0] < 0) != (mt[b, h, 1] < 0)) for b in used for h in range(N_KV))
+    assert mixed > 0, "no tile with exactly one raw side: pick another seed or slot size"
+    # free sequence 1: its tiles return to the stack and its mode entries are reset
+    blocks = torch.from_numpy(P.bt_cpu[1][:3].copy()).to(dev)
+    P.st.release_blocks(blocks)
+    torch.cuda.synchronize()
+    mt1 = P.st.mt.cpu().numpy().reshape(-1, 2 * N_KV)
+    for b in P.bt_cpu[1][:3]:
+        assert np.array_equal(mt1[b], np.arange(b * 2 * N_KV, (b + 1) * 2 * N_KV))
+    assert int(P.st.top) == 72 - int((P.st.mt < 0).sum())
+    assert sorted(P.st.stack[:int(P.st.top)].cpu().tolist() + [int(~m) for m in P.st.mt.cpu().tolist() if m < 0]) == list(range(72))
+
+
+def test_raw_pool_exhaustion_is_counted_not_written():
+    dev = require_gpu()
+    P = _Pool(dev, n_seq=2, max_blocks=4, num_blocks=8, raw_tiles=2 * N_KV)      # room for ONE filling block
+    P.step({0: _rows(5, 1), 1: _rows(3, 2)})
+    torch.cuda.synchronize()
+    assert int(P.st.err) == 2 * N_KV and int(P.st.top) == 0
+    with pytest.raises(RuntimeError, match="raw side pool exhausted"):
+        P.st.check()
+
+
+def test_bad_arguments_raise():
+    dev = require_gpu()
+    from gaac_amd.paged import LayerState
+    st = LayerState(8, N_KV, 8, _bases(dev), 128, dev)
+    buf = torch.zeros(LayerState.pool_bytes(8, N_KV), dtype=torch.uint8, device=dev)
+    q = torch.zeros(1, N_KV * G, 128, dtype=torch.bfloat16, device=dev)
+    bt = torch.zeros(1, 2, dtype=torch.int32, device=dev); sl = torch.ones(1, dtype=torch.int32, device=dev)
+    with pytest.raises(RuntimeError, match="max_seq_len"):
+        st.attention(q, buf, bt, sl, nsplit=1, max_seq_len=16 * 3)       # more blocks than the table holds
+    with pytest.raises(RuntimeError, match="GQA"):
+        st.attention(torch.zeros(1, N_KV * 17, 128, dtype=torch.bfloat16, device=dev), buf, bt, sl, nsplit=1)
