@@ -81,12 +81,16 @@ def main():
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="also run the library's plain 64 MiB copy kernel 10 times (the known-size kernel for scaling FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--cpu-heads", type=int, default=8, help="kv heads in the CPU baseline sample (0 = skip)")
+    ap.add_argument("--workload", default="decode64k", choices=["decode64k", "codec", "paged"],
+                    help="decode64k = the headline (config 1); codec = config 0 round trip; paged = config 3 serving step")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one MI355X; this build has no multi-GPU path (the hot path shards by kv head without any exchange). Use --gpus 1.", file=sys.stderr)
         sys.exit(2)
     if not torch.cuda.is_available():
         print("bench.py needs a GPU: the product has no CPU path.", file=sys.stderr); sys.exit(2)
+    if a.workload == "codec": return bench_codec(a)
+    if a.workload == "paged": return bench_paged(a)
     from gaac_amd import Codec, TileEncoder
     from gaac_amd.kernel import attn_launch, choose_nsplit, nsplit_with_tail_row, AttnWorkspace
     dev = "cuda"
@@ -202,6 +206,105 @@ def main():
     else:
         res["cpu_baseline"] = None
     print(json.dumps(res))
+
+
+def _median_us(fn, n, warm=5):
+    for _ in range(warm): fn()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+    for e0, e1 in evs:
+        e0.record(); fn(); e1.record()
+    torch.cuda.synchronize()
+    ts = sorted(e0.elapsed_time(e1) * 1e3 for e0, e1 in evs)
+    return ts[len(ts) // 2]
+
+
+def bench_codec(a):
+    """Config 0: K [8 kv heads, 4096 tokens, 128] seed 0, bases from the first 1024 tokens, encode as 256 tiles per head, decode."""
+    from gaac_amd import Codec, TileEncoder
+    from oracle import gaac_oracle as O
+    dev = "cuda"
+    x = make_kv(0, 8, 4096)
+    xd = x.to(dev)
+    codec = Codec(8).calibrate(xd[:, :1024])
+    enc = TileEncoder("k")
+    page = enc.encode(codec, xd)
+    back = Codec.decode(page)
+    exact = bool(torch.equal(back.view(torch.int16), xd.view(torch.int16)))
+    s3, s4, sr = tier_shares(page)
+    t_enc = _median_us(lambda: enc.encode(codec, xd), 30); t_dec = _median_us(lambda: Codec.decode(page), 30)
+    x16 = x.contiguous().view(torch.int16).numpy().view(np.uint16)
+    t0 = time.perf_counter()
+    b3, b4 = O.calibrate(x16[:, :1024], 8); op = O.encode(x16, "k", b3, b4, 8); t1 = time.perf_counter(); od = O.decode(op); t2 = time.perf_counter()
+    same = np.array_equal(od, x16) and int(op.ovf_head_start[-1]) == int(page.ovf_head_start[-1]) and np.array_equal(b3, codec.base3.cpu().numpy())
+    print(json.dumps({"workload": "config 0: codec round trip, K [8, 4096, 128] bf16", "ratio": round(page.ratio, 4), "tier_shares": [round(s3, 4), round(s4, 4), round(sr, 5)],
+                      "bit_exact": exact, "matches_cpu_oracle": bool(same), "encode_us": round(t_enc, 1), "decode_us": round(t_dec, 1),
+                      "encode_note": "TileEncoder.encode incl. its allocations and one host sync (sizes the escape stream)",
+                      "cpu_oracle_encode_ms": round((t1 - t0) * 1e3, 1), "cpu_oracle_decode_ms": round((t2 - t1) * 1e3, 1)}))
+
+
+def bench_paged(a):
+    """Config 3: 16 sequences, context lengths U{4096..65536} (seed 4), 32 q / 8 kv heads, block table = random permutation of the pool
+    (seed 5); every step stores one new token per sequence (blocks that fill up are compressed) and runs decode attention."""
+    from gaac_amd.codec import exponent_hist, bases_from_hist
+    from gaac_amd.paged import LayerState, build_store_entries, choose_nsplit, BLOCK
+    dev = "cuda"
+    n_seq, n_kv, n_q, steps = 16, N_KV, N_KV * G, max(32, min(a.steps, 64))
+    lens = np.random.default_rng(4).integers(4096, 65537, n_seq).tolist()
+    max_blocks = -(-(max(lens) + steps) // BLOCK)
+    need_blocks = sum(-(-(L + steps) // BLOCK) for L in lens)
+    perm = np.random.default_rng(5).permutation(need_blocks)
+    bt_cpu = np.zeros((n_seq, max_blocks), np.int32); o = 0
+    for i, L in enumerate(lens):
+        nb = -(-(L + steps) // BLOCK); bt_cpu[i, :nb] = perm[o:o + nb]; o += nb
+    g = torch.Generator(device=dev).manual_seed(6)
+    sig_k = torch.exp2(torch.rand(1, n_kv, D, generator=g, device=dev) * 8 - 4); sig_v = torch.exp2(torch.rand(1, n_kv, D, generator=g, device=dev) * 8 - 4)
+    def rows(n, sig):      # [n, n_kv, 128] bf16 with the distribution of config 0 (outlier per group with probability 0.002), made on the device
+        x = torch.randn(n, n_kv, D, generator=g, device=dev) * sig
+        hit = torch.rand(n, n_kv, D // 8, generator=g, device=dev) < 0.002
+        which = torch.randint(0, 8, (n, n_kv, D // 8), generator=g, device=dev)
+        boost = torch.ones(n, n_kv, D // 8, 8, device=dev).scatter_(-1, which.unsqueeze(-1), torch.where(hit, 4096.0, 1.0).unsqueeze(-1))
+        return (x * boost.view(n, n_kv, D)).to(torch.bfloat16)
+    cal_k, cal_v = rows(1024, sig_k), rows(1024, sig_v)
+    k3, k4 = bases_from_hist(exponent_hist(cal_k, n_kv), n_kv); v3, v4 = bases_from_hist(exponent_hist(cal_v, n_kv), n_kv)
+    raw_tiles = 2 * n_kv * 4 * n_seq + need_blocks * 2 * n_kv // 100 + 64
+    st = LayerState(need_blocks, n_kv, raw_tiles, dict(k3=k3, k4=k4, v3=v3, v4=v4), 128, dev)
+    buf = torch.zeros(LayerState.pool_bytes(need_blocks, n_kv), dtype=torch.uint8, device=dev)
+    for i, L in enumerate(lens):      # prompts
+        ent = build_store_entries([0], [L], [bt_cpu[i]])
+        st.store(rows(L, sig_k), rows(L, sig_v), buf, torch.from_numpy(ent).to(dev))
+    st.check()
+    bt = torch.from_numpy(bt_cpu).to(dev)
+    q = torch.randn(n_seq, n_q, D, generator=g, device=dev).to(torch.bfloat16)
+    nsplit = a.nsplit or choose_nsplit(n_seq, n_kv, max(lens) + steps)
+    cur = list(lens)
+    seq_lens = torch.tensor(cur, dtype=torch.int32, device=dev)
+    freeq = torch.empty(n_seq * 2 * n_kv, dtype=torch.int32, device=dev)
+    t_store, t_attn = [], []
+    for s in range(steps):
+        ent = torch.from_numpy(build_store_entries(cur, [1] * n_seq, bt_cpu)).to(dev)
+        kn, vn = rows(n_seq, sig_k), rows(n_seq, sig_v)
+        e = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+        e[0].record(); st.store(kn, vn, buf, ent, freeq); e[1].record()
+        cur = [c + 1 for c in cur]; seq_lens += 1
+        st.attention(q, buf, bt, seq_lens, nsplit, max_seq_len=max(cur)); e[2].record()
+        torch.cuda.synchronize()
+        t_store.append(e[0].elapsed_time(e[1]) * 1e3); t_attn.append(e[1].elapsed_time(e[2]) * 1e3)
+    st.check()
+    # bytes the attention has to read: full slots up to the used escape bytes, raw tiles in full
+    mt = st.mt.cpu().numpy().reshape(need_blocks, 2 * n_kv)
+    n_tiles = sum(-(-c // BLOCK) for c in cur) * 2 * n_kv
+    used_blocks = np.concatenate([bt_cpu[i, :-(-c // BLOCK)] for i, c in enumerate(cur)])
+    n_raw = int((mt[used_blocks] < 0).sum())
+    read_bytes = (n_tiles - n_raw) * 2880 + n_raw * 4096        # + escape bytes (about 1 % more): not counted
+    bf16_bytes = sum(cur) * n_kv * 2 * 256
+    pool_bytes = len(used_blocks) * 2 * n_kv * st.TS + n_raw * 4096
+    bf16_pool = len(used_blocks) * BLOCK * n_kv * 2 * 256
+    med = lambda v: sorted(v)[len(v) // 2]
+    print(json.dumps({"workload": "config 3: paged serving step, 16 sequences, 32 q / 8 kv heads, d=128", "context_tokens": sum(cur), "steps": steps, "nsplit": nsplit,
+                      "attention_us": round(med(t_attn), 1), "store_us": round(med(t_store), 1), "step_us": round(med(t_attn) + med(t_store), 1),
+                      "attention_read_GBps": round(read_bytes / med(t_attn) / 1e3, 1), "bf16_equivalent_GBps": round(bf16_bytes / med(t_attn) / 1e3, 1),
+                      "slot_pool_bytes": pool_bytes, "bf16_pool_bytes": bf16_pool, "pool_ratio": round(bf16_pool / pool_bytes, 4),
+                      "raw_tiles_in_use": n_raw, "tiles": n_tiles}))
 
 
 if __name__ == "__main__":

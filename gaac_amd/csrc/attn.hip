@@ -323,13 +323,11 @@ __device__ __forceinline__ void load_tile(const Bases& B, int tile, int lane, co
 struct WaveState { f32x4 acc[8]; float m_run, mu_run, l_run; };     // acc[i][r] = O[head a][group 4q+r, element i]; m in raw score units
 
 // unit decode with the escape contribution already expanded to exponent-field words x (see AttnLds::xlut)
-__device__ __forceinline__ void decode_unit_x(u32 slo, u32 shi, u32 g24, bool t0, const u32x4& x, const u32x4& b3w, const u32x4& b4w,
-                                              u32* __restrict__ out) {
+__device__ __forceinline__ void decode_unit_x(u32 slo, u32 shi, u32 g24, const u32x4& x, const u32x4& bw, u32* __restrict__ out) {
   const u32 cw = (g24 & 0xFFFu) | ((g24 << 4) & 0x0FFF0000u);
   const u32 c0 = (cw << 7) & 0x03800380u, c1 = (cw << 4) & 0x03800380u, c2 = (cw << 1) & 0x03800380u, c3 = (cw >> 2) & 0x03800380u;
-  // t0: 3-bit group (base3); otherwise base4 (raw groups: x already holds hi5 - base4)
-  const u32 e0 = c0 + (t0 ? b3w[0] : b4w[0]) + x[0], e1 = c1 + (t0 ? b3w[1] : b4w[1]) + x[1];
-  const u32 e2 = c2 + (t0 ? b3w[2] : b4w[2]) + x[2], e3 = c3 + (t0 ? b3w[3] : b4w[3]) + x[3];
+  // bw: the base words of the unit's tier (3-bit base, or 4-bit base for promoted and raw groups: their x holds hi5 - base4)
+  const u32 e0 = c0 + bw[0] + x[0], e1 = c1 + bw[1] + x[1], e2 = c2 + bw[2] + x[2], e3 = c3 + bw[3] + x[3];
   out[0] = (e0 & EXP_MASK2) | (__builtin_amdgcn_perm(shi, slo, 0x04040000u) & ~EXP_MASK2);
   out[1] = (e1 & EXP_MASK2) | (__builtin_amdgcn_perm(shi, slo, 0x05050101u) & ~EXP_MASK2);
   out[2] = (e2 & EXP_MASK2) | (__builtin_amdgcn_perm(shi, slo, 0x06060202u) & ~EXP_MASK2);
@@ -350,20 +348,26 @@ __device__ __forceinline__ u32x4 raw_x_words(u32 lo, u32 hi, const u32x4& b4w) {
 // group somewhere (most tiles, few lanes) patches those units from the prefetched bytes.  A lane with two or more raw groups
 // (its bytes may not fit the 8 prefetched ones) re-reads memory: only the SLOW instantiation contains those loads, so the
 // common instantiation has no memory access between the prefetch and the products.
+// bw[u]: the exponent-base words of unit u's tier, read from the block's LDS table: one table row per (tier, group), so the tier
+// select costs an address bit instead of four conditional moves per unit.
 template <int KIND, bool SLOW>
-__device__ __forceinline__ void unit_x_words(const KindRegs& R, const AttnLds& L, const uint8_t* __restrict__ esc_tile, int q,
-                                             const u32x4* __restrict__ b4w /* K: [4] per unit, V: [1] */, u32& tag8, u32x4* __restrict__ x) {
-  tag8 = __builtin_amdgcn_ubfe(R.f, 8 * q, 8);
+__device__ __forceinline__ void unit_x_words(const KindRegs& R, const AttnLds& L, const uint8_t* __restrict__ esc_tile, int a, int q,
+                                             u32x4* __restrict__ x, u32x4* __restrict__ bw) {
+  const u32 tag8 = __builtin_amdgcn_ubfe(R.f, 8 * q, 8);
   const u32 eb4 = __builtin_amdgcn_perm(R.e[1], R.e[0], L.sel[tag8]);
+  const u32x4* tab = KIND == KIND_K ? &L.bwk[0][4 * q] : &L.bwv[0][a];      // row of unit 0 at tier 0; tier 1 is NG rows further
 #pragma unroll
-  for (int u = 0; u < 4; ++u) x[u] = L.xlut[(eb4 >> (8 * u)) & 0xFFu];
+  for (int u = 0; u < 4; ++u) {
+    x[u] = L.xlut[(eb4 >> (8 * u)) & 0xFFu];
+    bw[u] = tab[(KIND == KIND_K ? u : 0) + NG * ((tag8 >> (2 * u)) & 1u)];
+  }
   if (__builtin_amdgcn_ballot_w64((tag8 & 0xAAu) != 0u)) {
     const u64 e64 = (u64)R.e[0] | ((u64)R.e[1] << 32);
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
       if (((tag8 >> (2 * u)) & 3u) == 3u) {          // offset = number of 4-bit groups below (a raw one below is handled next)
         const u64 v = e64 >> (8 * __popc(tag8 & (0x55u & ((1u << (2 * u)) - 1u))));
-        x[u] = raw_x_words((u32)v, (u32)(v >> 32), b4w[KIND == KIND_K ? u : 0]);
+        x[u] = raw_x_words((u32)v, (u32)(v >> 32), bw[u]);
       }
     }
     if (SLOW && __popc(tag8 & 0xAAu) >= 2) {
@@ -373,7 +377,7 @@ __device__ __forceinline__ void unit_x_words(const KindRegs& R, const AttnLds& L
         const u32 t = (tag8 >> (2 * u)) & 3u;
         if (t) {
           const u64 v = load_u64_unaligned(esc_tile + R.pos0 + off);
-          x[u] = t == 1u ? L.xlut[(u32)v & 0xFFu] : raw_x_words((u32)v, (u32)(v >> 32), b4w[KIND == KIND_K ? u : 0]);
+          x[u] = t == 1u ? L.xlut[(u32)v & 0xFFu] : raw_x_words((u32)v, (u32)(v >> 32), bw[u]);
         }
         off += (u32)tag_size(t);
       }
@@ -381,26 +385,22 @@ __device__ __forceinline__ void unit_x_words(const KindRegs& R, const AttnLds& L
   }
 }
 
-__device__ __forceinline__ bool tier0(u32 tag8, int u) { return (tag8 & (1u << (2 * u))) == 0u; }
-
 // PARTIAL: the tile is the last one of the sequence and only partly filled (rows >= S are masked out).  It is a template
 // parameter, not a run-time branch, so that no branch separates the score MFMAs from the first read of their result.
 template <bool PAGED, bool PARTIAL, bool SLOW>
 __device__ __forceinline__ void consume_tile(const TileRegs& R, WaveState& st, const AttnLds& L, const Bases& B,
                                              u32 kto, u32 vto, int tile, int S, float scale_log2e, int a, int q,
-                                             const u32x4 (&qf)[4], const u32x4 (&kb3)[4], const u32x4 (&kb4)[4],
-                                             const u32x4& vb3, const u32x4& vb4) {
-  u32 ktag8, vtag8;
-  u32x4 xk[4], xv[4];
-  unit_x_words<KIND_K, SLOW>(R.k, L, esc_of_tile<PAGED>(B.kov, kto, B.TS), q, kb4, ktag8, xk);
-  unit_x_words<KIND_V, SLOW>(R.v, L, esc_of_tile<PAGED>(B.vov, vto, B.TS), q, &vb4, vtag8, xv);
+                                             const u32x4 (&qf)[4]) {
+  u32x4 xk[4], xv[4], bk[4], bv[4];
+  unit_x_words<KIND_K, SLOW>(R.k, L, esc_of_tile<PAGED>(B.kov, kto, B.TS), a, q, xk, bk);
+  unit_x_words<KIND_V, SLOW>(R.v, L, esc_of_tile<PAGED>(B.vov, vto, B.TS), a, q, xv, bv);
   // ---- scores: S[tok 4q+r][head a]
   f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
     u32 slo, shi, w[4];
     unit_sm(R.k.pay, u, slo, shi);
-    decode_unit_x(slo, shi, unit_code_word(R.k.pay.c0, R.k.pay.c1, R.k.pay.c2, u), tier0(ktag8, u), xk[u], kb3[u], kb4[u], w);
+    decode_unit_x(slo, shi, unit_code_word(R.k.pay.c0, R.k.pay.c1, R.k.pay.c2, u), xk[u], bk[u], w);
     const u32x4 av = {w[0], w[1], w[2], w[3]};
     sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av), __builtin_bit_cast(bf16x8, qf[u]), sacc, 0, 0, 0);
   }
@@ -431,7 +431,7 @@ __device__ __forceinline__ void consume_tile(const TileRegs& R, WaveState& st, c
   for (int u = 0; u < 4; ++u) {
     u32 slo, shi;
     unit_sm(R.v.pay, u, slo, shi);
-    decode_unit_x(slo, shi, unit_code_word(R.v.pay.c0, R.v.pay.c1, R.v.pay.c2, u), tier0(vtag8, u), xv[u], vb3, vb4, W[u]);
+    decode_unit_x(slo, shi, unit_code_word(R.v.pay.c0, R.v.pay.c1, R.v.pay.c2, u), xv[u], bv[u], W[u]);
   }
   if (PARTIAL) {                // rows beyond the sequence must not reach the product
 #pragma unroll
@@ -451,13 +451,12 @@ __device__ __forceinline__ void consume_tile(const TileRegs& R, WaveState& st, c
 // A tile needs the SLOW instantiation when some lane holds two or more raw groups (about 1 tile in 100 at 0.3 % raw groups).
 template <bool PAGED, bool PARTIAL>
 __device__ __forceinline__ void consume(const TileRegs& R, WaveState& st, const AttnLds& L, const Bases& B, u32 kto, u32 vto, int tile,
-                                        int S, float scale_log2e, int a, int q, const u32x4 (&qf)[4], const u32x4 (&kb3)[4],
-                                        const u32x4 (&kb4)[4], const u32x4& vb3, const u32x4& vb4) {
+                                        int S, float scale_log2e, int a, int q, const u32x4 (&qf)[4]) {
   const u32 kr = __builtin_amdgcn_ubfe(R.k.f, 8 * q, 8) & 0xAAu, vr = __builtin_amdgcn_ubfe(R.v.f, 8 * q, 8) & 0xAAu;
   if (__builtin_expect(__builtin_amdgcn_ballot_w64(((kr & (kr - 1u)) | (vr & (vr - 1u))) != 0u) != 0, 0))
-    consume_tile<PAGED, PARTIAL, true>(R, st, L, B, kto, vto, tile, S, scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+    consume_tile<PAGED, PARTIAL, true>(R, st, L, B, kto, vto, tile, S, scale_log2e, a, q, qf);
   else
-    consume_tile<PAGED, PARTIAL, false>(R, st, L, B, kto, vto, tile, S, scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+    consume_tile<PAGED, PARTIAL, false>(R, st, L, B, kto, vto, tile, S, scale_log2e, a, q, qf);
 }
 
 // ---------------------------------------------------------------------------------------------------- main kernel
@@ -518,10 +517,9 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
   __syncthreads();        // block tables are ready
   // Q as the B operand of the score product: lane (head a, quad q), product u covers group 4q+u in word order (e, e+4);
   // exponent-base words of the lane's units
-  u32x4 qf[4], kb3[4], kb4[4];
+  u32x4 qf[4];
 #pragma unroll
-  for (int u = 0; u < 4; ++u) { qf[u] = L.qw[a][4 * q + u]; kb3[u] = L.bwk[0][4 * q + u]; kb4[u] = L.bwk[1][4 * q + u]; }
-  const u32x4 vb3 = L.bwv[0][a], vb4 = L.bwv[1][a];
+  for (int u = 0; u < 4; ++u) qf[u] = L.qw[a][4 * q + u];
 
   WaveState st;
 #pragma unroll
@@ -535,27 +533,27 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
       TgC1 = Tg;
       load_tile<PAGED>(B, t + 4, lane, Tg, R1);
       load_tags<PAGED>(B, TT, min(t + 8, tlast), a, Tg);
-      if (!PAGED || !TgC0.raw) consume<PAGED, false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+      if (!PAGED || !TgC0.raw) consume<PAGED, false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf);
       TgC0 = Tg;
       load_tile<PAGED>(B, t + 8, lane, Tg, R0);
       load_tags<PAGED>(B, TT, min(t + 12, tlast), a, Tg);
-      if (!PAGED || !TgC1.raw) consume<PAGED, false>(R1, st, L, B, TgC1.kto, TgC1.vto, t + 4, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+      if (!PAGED || !TgC1.raw) consume<PAGED, false>(R1, st, L, B, TgC1.kto, TgC1.vto, t + 4, S, A.scale_log2e, a, q, qf);
     }
     const int t = t0 + 4 * i;
     if (n - i == 2) {
       TgC1 = Tg;
       load_tile<PAGED>(B, t + 4, lane, Tg, R1);
-      if (!PAGED || !TgC0.raw) consume<PAGED, false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
-      if (!PAGED || !TgC1.raw) consume<PAGED, false>(R1, st, L, B, TgC1.kto, TgC1.vto, t + 4, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+      if (!PAGED || !TgC0.raw) consume<PAGED, false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf);
+      if (!PAGED || !TgC1.raw) consume<PAGED, false>(R1, st, L, B, TgC1.kto, TgC1.vto, t + 4, S, A.scale_log2e, a, q, qf);
     } else {
-      if (!PAGED || !TgC0.raw) consume<PAGED, false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+      if (!PAGED || !TgC0.raw) consume<PAGED, false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf);
     }
   }
   if (own_partial) {
     const int t = ntiles - 1;
     load_tags<PAGED>(B, TT, t, a, Tg);
     load_tile<PAGED>(B, t, lane, Tg, R0);
-    if (!PAGED || !Tg.raw) consume<PAGED, true>(R0, st, L, B, Tg.kto, Tg.vto, t, S, A.scale_log2e, a, q, qf, kb3, kb4, vb3, vb4);
+    if (!PAGED || !Tg.raw) consume<PAGED, true>(R0, st, L, B, Tg.kto, Tg.vto, t, S, A.scale_log2e, a, q, qf);
   }
   // ---- rows kept as plain BF16: the raw tail of a cache head (the extra block row) or, in the paged pool, tiles of this split
   // whose K or V side is a raw tile (the block that is still filling, or escapes that did not fit the slot)
