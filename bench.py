@@ -168,19 +168,34 @@ def main():
     ts = sorted(e0.elapsed_time(e1) * 1e3 / BATCH for e0, e1 in evs)
     split_us_mean, split_us_med = sum(ts) / len(ts), ts[len(ts) // 2]
 
-    # ---- uncompressed BF16 decode attention on the same GPU (torch SDPA over the same tokens), rotating copies
-    kb = [torch.cat([kd], 1).view(1, H, S_CTX + TAIL_TOK, D).clone() for _ in range(a.copies)]
-    vb = [vd.view(1, H, S_CTX + TAIL_TOK, D).clone() for _ in range(a.copies)]
+    # ---- uncompressed BF16 decode attention on the same GPU over the same tokens (compressed part + tail, contiguous), rotating copies:
+    # (a) the library's own baseline kernel = this kernel's structure without the decoder, best of a few split counts;
+    # (b) torch's scaled_dot_product_attention, for reference only
+    from gaac_amd.kernel import bf16_attention
+    kb = [kd.clone() for _ in range(a.copies)]; vb = [vd.clone() for _ in range(a.copies)]
+    qb = qd.view(1, n_q, D)
+    ref_b = bf16_attention(qb, kb[0], vb[0], scale).float().view(n_q, D)
+    assert (ref_b - ref).abs().max().item() <= 1e-2, "baseline kernel is off"
+    bf16_us, bf16_ns = None, None
+    for ns in (64, 96, 128, 192):
+        wsb = AttnWorkspace(n_q, ns, torch.bfloat16, dev)
+        for i in range(10): bf16_attention(qb, kb[i % a.copies], vb[i % a.copies], scale, ns, wsb)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        n_b = max(60, a.steps // 2)
+        e0.record()
+        for i in range(n_b): bf16_attention(qb, kb[i % a.copies], vb[i % a.copies], scale, ns, wsb)
+        e1.record(); torch.cuda.synchronize()
+        t = e0.elapsed_time(e1) * 1e3 / n_b
+        if bf16_us is None or t < bf16_us: bf16_us, bf16_ns = t, ns
     q4 = qd.view(1, n_q, 1, D)
-    sdpa = lambda i: torch.nn.functional.scaled_dot_product_attention(q4, kb[i % a.copies], vb[i % a.copies], scale=scale, enable_gqa=True)
-    for i in range(10): sdpa(i)
-    torch.cuda.synchronize()
+    k4 = [x.view(1, H, S_CTX + TAIL_TOK, D) for x in kb]; v4 = [x.view(1, H, S_CTX + TAIL_TOK, D) for x in vb]
+    sdpa = lambda i: torch.nn.functional.scaled_dot_product_attention(q4, k4[i % a.copies], v4[i % a.copies], scale=scale, enable_gqa=True)
+    for i in range(3): sdpa(i)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    n_b = max(20, a.steps // 5)
     e0.record()
-    for i in range(n_b): sdpa(i)
+    for i in range(10): sdpa(i)
     e1.record(); torch.cuda.synchronize()
-    bf16_us = e0.elapsed_time(e1) * 1e3 / n_b
+    sdpa_us = e0.elapsed_time(e1) * 1e3 / 10
 
     s3k, s4k, srk = tier_shares(kp); s3v, s4v, srv = tier_shares(vp)
     res = {
@@ -193,7 +208,9 @@ def main():
         "compression_ratio_k": round(kp.ratio, 4), "compression_ratio_v": round(vp.ratio, 4),
         "tier_shares_k": [round(s3k, 4), round(s4k, 4), round(srk, 5)], "tier_shares_v": [round(s3v, 4), round(s4v, 4), round(srv, 5)],
         "check": {"vs": "fp32 softmax attention (torch, device) over HIP-decoded KV", "max_abs": err_max, "mean_abs": err_mean, "roundtrip_bit_exact": True},
-        "bf16_sdpa_us": round(bf16_us, 2), "speedup_vs_bf16_sdpa": round(bf16_us / us_step, 3),
+        "bf16_baseline": {"kernel": "k_bf16_attn_split (same structure, no decoder)", "us": round(bf16_us, 2), "nsplit": bf16_ns,
+                          "GBps": round(bf16_bytes / bf16_us / 1e3, 1), "speedup_of_compressed": round(bf16_us / us_step, 3),
+                          "torch_sdpa_us": round(sdpa_us, 1)},
         "roofline": {"bound": "hbm", "achieved": round(alg_bytes / split_us_mean / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(alg_bytes / split_us_mean / 1e3 / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC["bytes"] if nsplit == MEASURED_TRAFFIC["nsplit"] else None,

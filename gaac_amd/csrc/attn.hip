@@ -669,6 +669,138 @@ __global__ void __launch_bounds__(512) k_attn_combine(const float* __restrict__ 
   }
 }
 
+// ---------------------------------------------------------------------------------------------------- uncompressed baseline
+// Decode attention over plain BF16 K/V [cache head][token][128] with the same structure as k_attn_split (same split / wave / MFMA
+// mapping, online softmax, block merge and fused last-block merge) minus the decoder: the baseline the compressed path is compared
+// with on the same GPU.  Args reuse AttnArgs: kt / vt = K / V, S_pad = token stride of a head, tcap = tokens per head.
+struct RawTile { u32x4 k[4], v[4]; };
+// K: lane (token a, quad q) holds channels 32 j + 8 q .. + 8 for product j.  V: lane (a, q) holds channels 8 a .. 8 a + 8 of tokens 4 q + r.
+__device__ __forceinline__ void load_raw_tile(const u16* __restrict__ kh, const u16* __restrict__ vh, int tile, int S, int a, int q, RawTile& R) {
+  const int kt = min(tile * T + a, S - 1);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) R.k[j] = *reinterpret_cast<const u32x4*>(kh + (long)kt * D + 32 * j + 8 * q);
+#pragma unroll
+  for (int r = 0; r < 4; ++r) R.v[r] = *reinterpret_cast<const u32x4*>(vh + (long)min(tile * T + 4 * q + r, S - 1) * D + 8 * a);
+}
+template <bool PARTIAL>
+__device__ __forceinline__ void consume_raw_tile(const RawTile& R, WaveState& st, int tile, int S, float scale_log2e, int q, const u32x4 (&qf)[4]) {
+  f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, R.k[j]), __builtin_bit_cast(bf16x8, qf[j]), sacc, 0, 0, 0);
+  const int tok0 = tile * T + 4 * q;
+  if (PARTIAL) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) sacc[r] = tok0 + r >= S ? -INFINITY : sacc[r];
+  }
+  const float tmax = quad_rows_max(fmaxf(fmaxf(sacc[0], sacc[1]), fmaxf(sacc[2], sacc[3])));
+  if (__builtin_amdgcn_ballot_w64(tmax > st.m_run)) {
+    const float mn = fmaxf(st.m_run, tmax), mu = mn == -INFINITY ? 0.f : mn * scale_log2e;
+    const float alpha = __builtin_amdgcn_exp2f(st.m_run == -INFINITY ? -INFINITY : st.mu_run - mu);
+    st.l_run *= alpha;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) st.acc[i] *= alpha;
+    st.m_run = mn; st.mu_run = mu;
+  }
+  float p[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) p[r] = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[r], scale_log2e, -st.mu_run));
+  st.l_run += (p[0] + p[1]) + (p[2] + p[3]);
+  const u32x2 pw = {pack_bf16x2(p[0], p[1]), pack_bf16x2(p[2], p[3])};
+  const s16x4 pb = __builtin_bit_cast(s16x4, pw);
+#pragma unroll
+  for (int m = 0; m < 4; ++m) {      // word m of a row = channels 8 a + 2 m, + 1
+    u32 w[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) w[r] = PARTIAL && tok0 + r >= S ? 0u : R.v[r][m];
+    const u32x2 lo = {__builtin_amdgcn_perm(w[1], w[0], 0x05040100u), __builtin_amdgcn_perm(w[3], w[2], 0x05040100u)};
+    const u32x2 hi = {__builtin_amdgcn_perm(w[1], w[0], 0x07060302u), __builtin_amdgcn_perm(w[3], w[2], 0x07060302u)};
+    st.acc[2 * m] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, lo), pb, st.acc[2 * m], 0, 0, 0);
+    st.acc[2 * m + 1] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, hi), pb, st.acc[2 * m + 1], 0, 0, 0);
+  }
+}
+
+struct Bf16Lds { u32x4 qw[GMAX][NG]; float m[4][GMAX], l[4][GMAX]; float acc[4][GMAX][D]; };
+__global__ void __launch_bounds__(256, 2) k_bf16_attn_split(const AttnArgs A) {
+  __shared__ Bf16Lds L;
+  const int bh = blockIdx.x, split = blockIdx.y, tid = threadIdx.x;
+  const int b = bh / A.n_kv, kvh = bh % A.n_kv, G = A.G;
+  const long qh0 = (long)b * A.n_q + (long)kvh * G;
+  const int S = A.tcap;
+  const int ntiles = (S + T - 1) / T, chunk = (ntiles + A.nsplit - 1) / A.nsplit;
+  const int tlo = min(split * chunk, ntiles), thi = min(tlo + chunk, ntiles);
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, a = lane & 15, q = lane >> 4;
+  const u16* kh = A.kt + (long)bh * A.S_pad * D; const u16* vh = A.vt + (long)bh * A.S_pad * D;
+  const int t0 = tlo + wave;
+  const int n_all = t0 < thi ? (thi - t0 + 3) / 4 : 0;
+  const bool own_partial = n_all > 0 && (S % T) != 0 && t0 + 4 * (n_all - 1) == ntiles - 1;
+  const int n = n_all - (own_partial ? 1 : 0);
+  RawTile R0, R1;
+  if (n > 0) load_raw_tile(kh, vh, t0, S, a, q, R0);
+  // Q as the B operand: lane (head a, quad q), product j covers channels 32 j + 8 q .. + 8 (rows >= G are zero)
+  for (int i = tid; i < GMAX * NG; i += 256) {
+    const int h = i >> 4, c = i & 15;
+    L.qw[h][c] = h < G ? *reinterpret_cast<const u32x4*>(A.q + (qh0 + h) * D + 8 * c) : u32x4{0u, 0u, 0u, 0u};
+  }
+  __syncthreads();
+  u32x4 qf[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) qf[j] = L.qw[a][4 * j + q];
+  WaveState st;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) st.acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  st.m_run = -INFINITY; st.mu_run = 0.f; st.l_run = 0.f;
+  if (n > 0) {
+    int i = 0;
+    for (; i + 2 < n; i += 2) {
+      const int t = t0 + 4 * i;
+      load_raw_tile(kh, vh, t + 4, S, a, q, R1);
+      consume_raw_tile<false>(R0, st, t, S, A.scale_log2e, q, qf);
+      load_raw_tile(kh, vh, t + 8, S, a, q, R0);
+      consume_raw_tile<false>(R1, st, t + 4, S, A.scale_log2e, q, qf);
+    }
+    const int t = t0 + 4 * i;
+    if (n - i == 2) {
+      load_raw_tile(kh, vh, t + 4, S, a, q, R1);
+      consume_raw_tile<false>(R0, st, t, S, A.scale_log2e, q, qf);
+      consume_raw_tile<false>(R1, st, t + 4, S, A.scale_log2e, q, qf);
+    } else {
+      consume_raw_tile<false>(R0, st, t, S, A.scale_log2e, q, qf);
+    }
+  }
+  if (own_partial) {
+    load_raw_tile(kh, vh, ntiles - 1, S, a, q, R0);
+    consume_raw_tile<true>(R0, st, ntiles - 1, S, A.scale_log2e, q, qf);
+  }
+  asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");
+  const float l_run = quad_rows_sum(st.l_run);
+  const float m_run = st.m_run == -INFINITY ? -INFINITY : st.mu_run;
+  if (a < G) {
+    if (q == 0) { L.m[wave][a] = m_run; L.l[wave][a] = l_run; }
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) L.acc[wave][a][8 * (4 * q + r) + i] = st.acc[i][r];
+  }
+  __syncthreads();
+  const int d = tid & 127;
+  for (int g = tid >> 7; g < G; g += 2) {
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) M = fmaxf(M, L.m[w][g]);
+    float Lc = 0.f, Ac = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      const float f = L.m[w][g] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(L.m[w][g] - M);
+      Lc += L.l[w][g] * f; Ac += L.acc[w][g][d] * f;
+    }
+    const long pidx = (qh0 + g) * A.nslot + split;
+    if (d == 0) { store_partial(A.pm + pidx, M); store_partial(A.pl + pidx, Lc); }
+    store_partial(A.pa + pidx * D + d, Ac);
+  }
+  publish_and_merge(A, bh, qh0, G, tid, &L.acc[0][0][0]);
+}
+
 }  // namespace gaac
 
 using namespace gaac;
@@ -762,4 +894,19 @@ extern "C" int gaac_paged_attn(
   A.pool = pool; A.raw = (const u16*)raw; A.mt = mt; A.bt = bt; A.bt_stride = bt_stride; A.TS = TS;
   hipLaunchKernelGGL(k_attn_split<true>, dim3(B * n_kv, nsplit), dim3(256), 0, (hipStream_t)stream, A);
   return launch_status("gaac_paged_attn");
+}
+
+extern "C" int gaac_bf16_attn(const void* k, const void* v, int S, long head_stride_tokens, const void* q, int B, int n_q, int n_kv,
+                              float scale, int nsplit, float* pm, float* pl, float* pa, int* tickets, void* out, void* stream) {
+  GAAC_REQUIRE(n_kv > 0 && n_q > 0 && n_q % n_kv == 0 && n_q / n_kv <= GMAX, "GQA group size must be 1..%d (n_q=%d, n_kv=%d)", GMAX, n_q, n_kv);
+  GAAC_REQUIRE(k && v && q && pm && pl && pa && tickets && out, "gaac_bf16_attn: null pointer");
+  GAAC_REQUIRE(B > 0 && S > 0 && head_stride_tokens >= S && nsplit >= 1 && nsplit <= MAX_SLOTS, "gaac_bf16_attn: bad sizes");
+  AttnArgs A = {};
+  A.q = (const u16*)q; A.pm = pm; A.pl = pl; A.pa = pa;
+  A.S_pad = (int)head_stride_tokens; A.scale_log2e = scale * 1.4426950408889634f; A.nsplit = nsplit; A.nslot = nsplit;
+  A.n_kv = n_kv; A.n_q = n_q; A.G = n_q / n_kv; A.NB = 1;
+  A.kt = (const u16*)k; A.vt = (const u16*)v; A.tcap = S;
+  A.tickets = tickets; A.out = (u16*)out;
+  hipLaunchKernelGGL(k_bf16_attn_split, dim3(B * n_kv, nsplit), dim3(256), 0, (hipStream_t)stream, A);
+  return launch_status("gaac_bf16_attn");
 }

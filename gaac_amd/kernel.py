@@ -93,3 +93,17 @@ def attention(q, kp, vp, scale=None, nsplit=None, phase="fused"):
     out = attn_launch(kp, vp, q.reshape(B * n_q, Dq).contiguous(), slots, n_q, n_kv, SL, kp.sm.shape[1] // D,
                       scale if scale is not None else Dq ** -0.5, nsplit, phase=phase)
     return out.view(B, n_q, Dq)
+
+
+def bf16_attention(q, k, v, scale=None, nsplit=None, ws=None):
+    """Baseline: decode attention over UNCOMPRESSED K/V (k, v: [B*n_kv, S, D] bf16 contiguous; q: [B, n_q, D]) with the kernel
+    structure of the compressed path minus the decoder.  Returns [B, n_q, D] bf16."""
+    B, n_q, Dq = q.shape
+    H, S, _ = k.shape
+    n_kv = H // B
+    if nsplit is None: nsplit = choose_nsplit(B, n_kv, S)
+    if ws is None: ws = AttnWorkspace(B * n_q, nsplit, q.dtype, q.device)
+    p = _lib.ptr
+    _lib.call("gaac_bf16_attn", p(k), p(v), S, k.stride(0) // D, p(q.contiguous()), B, n_q, n_kv, float(scale if scale is not None else Dq ** -0.5),
+              nsplit, p(ws.pm), p(ws.pl), p(ws.pa), p(ws.tickets), p(ws.out), _lib.stream())
+    return ws.out.view(B, n_q, Dq)

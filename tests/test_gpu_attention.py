@@ -74,6 +74,20 @@ def test_fused_merge_equals_the_two_kernel_launch_and_rearms_its_tickets():
         assert int(ws.tickets.abs().sum().item()) == 0
 
 
+@pytest.mark.parametrize("B,n_kv,G,S", [(1, 8, 4, 4096), (2, 2, 16, 1000), (3, 2, 1, 16), (1, 4, 6, 333)])
+def test_uncompressed_baseline_kernel(B, n_kv, G, S):
+    """The BF16 baseline kernel (same structure, no decoder) against the same oracle and tolerance."""
+    dev = require_gpu()
+    from gaac_amd.kernel import bf16_attention
+    k16, v16 = kv_like16(B * n_kv, S, seed=21), kv_like16(B * n_kv, S, seed=22)
+    q16 = randn_bf16((B, n_kv * G, 128), seed=7, scale=0.1)
+    for ns in (None, 1, 5):
+        out = bf16_attention(to_bf16(q16, dev), to_bf16(k16, dev), to_bf16(v16, dev), SCALE, nsplit=ns)
+        got = O.bf16_to_f32(to_u16(out)); ref = _ref(q16, k16, v16, B, n_kv)
+        for b in range(B):
+            assert np.abs(got[b] - ref[b]).max() <= 2e-2 * np.abs(ref[b]).max() + 1e-3, (b, ns)
+
+
 def test_stated_tolerance_on_unit_scale_data():
     """max-abs <= 1e-2 and mean-abs <= 1e-3 against decompress + fp32 softmax attention, q ~ N(0,1)."""
     dev = require_gpu()
