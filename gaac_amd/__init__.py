@@ -4,5 +4,6 @@ from .codec import Codec, Page
 from .encoder import TileEncoder
 from .kernel import attention, choose_nsplit
 from .kv_cache import CompressedKVCache
+from .calibration import BaseCollector
 
-__all__ = ["Codec", "Page", "TileEncoder", "attention", "choose_nsplit", "CompressedKVCache"]
+__all__ = ["Codec", "Page", "TileEncoder", "attention", "choose_nsplit", "CompressedKVCache", "BaseCollector"]

@@ -104,3 +104,30 @@ def test_row_offsets_matches_oracle():
     flags = (tags << (2 * np.arange(16))).sum(-1).astype(np.uint32).view(np.int32)
     got = row_offsets(torch.from_numpy(flags).to(dev), 690)
     assert np.array_equal(got.cpu().numpy(), O.row_offsets(flags, 690))
+
+
+def test_base_collector_accumulates_over_steps_and_round_trips_its_file(tmp_path):
+    """BaseCollector (calibration.py of the reference): histograms add up over prefill steps; bases equal the oracle's on the
+    concatenated tokens; the saved file holds {layer: {k3,k4,v3,v4}} uint8 [n_kv,128] CPU tables and loads with weights_only."""
+    dev = require_gpu()
+    from gaac_amd import BaseCollector
+    from gaac_amd.calibration import load_bases
+    n_kv = 2
+    col = BaseCollector()
+    parts = {0: [], 1: []}
+    for step in range(3):
+        for layer in (0, 1):
+            k16 = np.ascontiguousarray(kv_like16(n_kv, 100 + 37 * step, seed=10 * step + layer).transpose(1, 0, 2))
+            v16 = np.ascontiguousarray(kv_like16(n_kv, 100 + 37 * step, seed=50 + 10 * step + layer).transpose(1, 0, 2))
+            col.observe(layer, to_bf16(k16, dev), to_bf16(v16, dev)); parts[layer].append((k16, v16))
+    path = str(tmp_path / "bases.pt")
+    assert col.save(path) == 2
+    tables = load_bases(path)
+    assert sorted(tables) == [0, 1]
+    for layer in (0, 1):
+        kall = np.concatenate([p[0] for p in parts[layer]]); vall = np.concatenate([p[1] for p in parts[layer]])
+        k3, k4 = O.bases_from_hist(O.exponent_hist(kall, n_kv), n_kv); v3, v4 = O.bases_from_hist(O.exponent_hist(vall, n_kv), n_kv)
+        t = tables[layer]
+        assert all(t[n].dtype == torch.uint8 and tuple(t[n].shape) == (n_kv, 128) and not t[n].is_cuda for n in ("k3", "k4", "v3", "v4"))
+        assert np.array_equal(t["k3"].numpy(), k3) and np.array_equal(t["k4"].numpy(), k4)
+        assert np.array_equal(t["v3"].numpy(), v3) and np.array_equal(t["v4"].numpy(), v4)
