@@ -115,8 +115,9 @@ __device__ __forceinline__ void merge_head_by_wave(const AttnArgs& A, long row, 
     *reinterpret_cast<u32x2*>(A.out + row * D + dq) = o;
   }
 }
-// Called by all 256 threads of a block after its partial has been written with store_partial().
-// fs: 4 x MAX_SLOTS floats of LDS that nothing else uses any more.
+// Called by all threads of a block (NW waves) after its partial has been written with store_partial().
+// fs: NW x MAX_SLOTS floats of LDS that nothing else uses any more.
+template <int NW>
 __device__ __forceinline__ void publish_and_merge(const AttnArgs& A, int bh, long qh0, int G, int tid, float* __restrict__ fs) {
   __shared__ int last;
   if (!A.tickets) return;
@@ -126,13 +127,13 @@ __device__ __forceinline__ void publish_and_merge(const AttnArgs& A, int bh, lon
   __syncthreads();
   if (!last) return;
   const int wave = tid >> 6, lane = tid & 63;
-  for (int g = wave; g < G; g += 4) merge_head_by_wave(A, qh0 + g, fs + wave * MAX_SLOTS, lane);
+  for (int g = wave; g < G; g += NW) merge_head_by_wave(A, qh0 + g, fs + wave * MAX_SLOTS, lane);
   if (tid == 0) __hip_atomic_store(&A.tickets[bh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);      // re-arm for the next launch
 }
 
 // ---------------------------------------------------------------------------------------------------- uncompressed rows
 // Attention of the block's G query heads over up to 16 rows kept as plain BF16 (the raw tail of a cache head, gaac_tail of
-// /root/reference/gaac/kernel.py:220-279), done by all 256 threads in fp32 on the VALU.  The result is folded into the running
+// /root/reference/gaac/kernel.py:220-279), done by the block's first 256 threads in fp32 on the VALU (all threads take part in the barriers).  The result is folded into the running
 // partial (m, l, acc) that the block merge treats as a fifth wave; several calls accumulate (online softmax).
 struct RawScratch {              // lives in the block-merge buffer, which is idle until the waves have finished their tiles
   float qs[GMAX][D];             // the query heads in fp32, natural channel order
@@ -140,10 +141,12 @@ struct RawScratch {              // lives in the block-merge buffer, which is id
   float alpha[GMAX];             // rescale factor of the running partial
   u16 krows[T * D], vrows[T * D];   // a compressed tile decoded next to a raw one (paged mode: only one kind of a tile is raw)
 };
+template <int NT>
 __device__ __forceinline__ void raw_rows_begin(RawScratch& R, const AttnArgs& A, long qh0, int G, int tid) {
-  for (int i = tid; i < G * D; i += 256) R.qs[i >> 7][i & 127] = bf16_bits_to_float(A.q[qh0 * D + i]);
+  for (int i = tid; i < G * D; i += NT) R.qs[i >> 7][i & 127] = bf16_bits_to_float(A.q[qh0 * D + i]);
 }
 // krows / vrows: 16 x 128 BF16, row stride D; rows >= nvalid are ignored.  m5/l5/acc5: the running partial [GMAX], [GMAX], [GMAX][D].
+template <int NT>
 __device__ __forceinline__ void raw_rows_attend(RawScratch& R, const u16* __restrict__ krows, const u16* __restrict__ vrows, int nvalid,
                                                 float scale_log2e, int G, int tid, float* __restrict__ m5, float* __restrict__ l5,
                                                 float (*__restrict__ acc5)[D]) {
@@ -152,7 +155,7 @@ __device__ __forceinline__ void raw_rows_attend(RawScratch& R, const u16* __rest
   float kr[8];
   {
     u32x4 kv = {0u, 0u, 0u, 0u};
-    if (t < nvalid) kv = *reinterpret_cast<const u32x4*>(krows + t * D + 8 * c);
+    if (t < nvalid && t < T) kv = *reinterpret_cast<const u32x4*>(krows + t * D + 8 * c);
 #pragma unroll
     for (int i = 0; i < 4; ++i) { kr[2 * i] = bf16_bits_to_float(kv[i] & 0xFFFFu); kr[2 * i + 1] = bf16_bits_to_float(kv[i] >> 16); }
   }
@@ -162,7 +165,7 @@ __device__ __forceinline__ void raw_rows_attend(RawScratch& R, const u16* __rest
     for (int i = 0; i < 8; ++i) d += R.qs[g][8 * c + i] * kr[i];
 #pragma unroll
     for (int o = 8; o > 0; o >>= 1) d += __shfl_xor(d, o, 16);
-    if (c == 0) R.sc[g][t] = t < nvalid ? d * scale_log2e : -INFINITY;
+    if (c == 0 && t < T) R.sc[g][t] = t < nvalid ? d * scale_log2e : -INFINITY;
   }
   __syncthreads();
   {   // thread (g = tid >> 4, token = tid & 15): softmax over the 16 lanes of the row, merged into the running partial
@@ -187,7 +190,7 @@ __device__ __forceinline__ void raw_rows_attend(RawScratch& R, const u16* __rest
   }
   __syncthreads();
   const int d = tid & 127;
-  for (int g = tid >> 7; g < G; g += 2) {
+  for (int g = tid >> 7; g < G; g += NT / 128) {
     float acc = acc5[g][d] * R.alpha[g];
     for (int tk = 0; tk < nvalid; ++tk) acc += R.sc[g][tk] * bf16_bits_to_float(vrows[tk * D + d]);
     acc5[g][d] = acc;
@@ -205,10 +208,11 @@ struct AttnLds {
   u32 sel[256];
   u32x4 bwk[2][NG], bwv[2][NG];
   u32x4 qw[GMAX][NG];
-  float m[5][GMAX], l[5][GMAX];   // per-wave partials of the block merge; [4] = the uncompressed rows
-  float acc[5][GMAX][D];          // acc[0..3] double as RawScratch before the waves publish and as the merge factors afterwards
 };
-static_assert(sizeof(RawScratch) <= 4 * GMAX * D * sizeof(float) && 4 * MAX_SLOTS <= 4 * GMAX * D, "scratch views must fit acc[0..3]");
+// Block merge: one partial per wave plus one (index NW) for the uncompressed rows.  acc[0..3] double as RawScratch before the waves
+// publish, acc[0..NW-1] as the merge factors afterwards.
+template <int NW> struct MergeLds { float m[NW + 1][GMAX], l[NW + 1][GMAX]; float acc[NW + 1][GMAX][D]; };
+static_assert(sizeof(RawScratch) <= 4 * GMAX * D * sizeof(float) && MAX_SLOTS <= GMAX * D, "scratch views must fit the merge buffer");
 struct TableRegs { u32 b0, b1; u32 qlo[4], qhi[4]; };      // one thread's raw inputs of the per-block tables
 // global loads only (issued before the first tile's loads so that the two latencies overlap)
 __device__ __forceinline__ void tables_load(TableRegs& Tr, int tid, const AttnArgs& A, int brow, long qh0) {
@@ -460,9 +464,12 @@ __device__ __forceinline__ void consume(const TileRegs& R, WaveState& st, const 
 }
 
 // ---------------------------------------------------------------------------------------------------- main kernel
-template <bool PAGED>
-__global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
+// NW = waves per block: 4 (two blocks per CU) or 8 (one block per CU: half as many partials to merge for the same occupancy)
+template <bool PAGED, int NW>
+__global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const AttnArgs A) {
+  constexpr int NT = 64 * NW;
   __shared__ AttnLds L;
+  __shared__ MergeLds<NW> M;
   __shared__ int2 tile_table[PAGED ? MAX_CHUNK : 1];
   const int bh = blockIdx.x, tid = threadIdx.x;
   // with a raw tail the grid has one more block row: it is dispatched first (blockIdx.y == 0), owns no compressed tile and writes
@@ -472,7 +479,7 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
   const int slot = PAGED ? 0 : A.slot[b], ch = PAGED ? kvh : (slot < 0 ? 0 : slot) * A.n_kv + kvh;
   const long qh0 = (long)b * A.n_q + (long)kvh * G;
   TableRegs Tr;
-  tables_load(Tr, tid, A, ch % A.NB, qh0);
+  if (tid < 256) tables_load(Tr, tid, A, ch % A.NB, qh0);
 
   const int S = PAGED ? max(A.sl[b], 0) : (slot < 0 ? 0 : A.sl[ch]);
   const int ntiles = (S + T - 1) / T, chunk = PAGED ? min((ntiles + A.nsplit - 1) / A.nsplit, MAX_CHUNK) : (ntiles + A.nsplit - 1) / A.nsplit;
@@ -484,7 +491,7 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
     // logical tile -> block table -> mode table (paged_kernel.py:137-138), resolved once per block into LDS
     B.kov = B.vov = A.pool; B.TS = A.TS;
     B.ksm = B.kcd = B.vsm = B.vcd = nullptr; B.kfl = B.kto = B.vfl = B.vto = nullptr;
-    for (int i = tid; i < thi - tlo; i += 256) {
+    for (int i = tid; i < thi - tlo; i += NT) {
       const long pc = (long)A.bt[(long)b * A.bt_stride + tlo + i] * (2 * A.n_kv) + 2 * kvh;
       tile_table[i] = int2{A.mt[pc], A.mt[pc + 1]};
     }
@@ -496,24 +503,24 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
     B.TS = 0;
   }
 
-  // tiles of this wave: t(i) = tlo + wave + 4 i, i < n.  Ping-pong registers R0/R1; tag words are fetched one tile further
+  // tiles of this wave: t(i) = tlo + wave + NW i, i < n.  Ping-pong registers R0/R1; tag words are fetched one tile further
   // ahead (index clamped to the wave's last tile, so that no load sits under a branch the consumer has to join).  A partly
   // filled last tile of the sequence is taken out of the pipeline and handled at the end by the wave that owns it.
   const int t0 = tlo + wave;
-  const int n_all = t0 < thi ? (thi - t0 + 3) / 4 : 0;
-  const bool own_partial = n_all > 0 && (S % T) != 0 && t0 + 4 * (n_all - 1) == ntiles - 1;
+  const int n_all = t0 < thi ? (thi - t0 + NW - 1) / NW : 0;
+  const bool own_partial = n_all > 0 && (S % T) != 0 && t0 + NW * (n_all - 1) == ntiles - 1;
   const int n = n_all - (own_partial ? 1 : 0);
-  const int tlast = t0 + 4 * (n - 1);
+  const int tlast = t0 + NW * (n - 1);
   TileRegs R0, R1;
   TagRegs Tg, TgC0, TgC1;
   if (n > 0) {          // start the first tile's loads before waiting for the block tables
     load_tags<PAGED>(B, TT, t0, a, Tg);
     TgC0 = Tg;
     load_tile<PAGED>(B, t0, lane, Tg, R0);
-    load_tags<PAGED>(B, TT, min(t0 + 4, tlast), a, Tg);
+    load_tags<PAGED>(B, TT, min(t0 + NW, tlast), a, Tg);
   }
-  tables_store(L, Tr, tid);
-  if (tid < GMAX) { L.m[4][tid] = -INFINITY; L.l[4][tid] = 0.f; }
+  if (tid < 256) tables_store(L, Tr, tid);
+  if (tid < GMAX) { M.m[NW][tid] = -INFINITY; M.l[NW][tid] = 0.f; }
   __syncthreads();        // block tables are ready
   // Q as the B operand of the score product: lane (head a, quad q), product u covers group 4q+u in word order (e, e+4);
   // exponent-base words of the lane's units
@@ -529,22 +536,22 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
   if (n > 0) {
     int i = 0;
     for (; i + 2 < n; i += 2) {
-      const int t = t0 + 4 * i;
+      const int t = t0 + NW * i;
       TgC1 = Tg;
-      load_tile<PAGED>(B, t + 4, lane, Tg, R1);
-      load_tags<PAGED>(B, TT, min(t + 8, tlast), a, Tg);
+      load_tile<PAGED>(B, t + NW, lane, Tg, R1);
+      load_tags<PAGED>(B, TT, min(t + 2 * NW, tlast), a, Tg);
       if (!PAGED || !TgC0.raw) consume<PAGED, false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf);
       TgC0 = Tg;
-      load_tile<PAGED>(B, t + 8, lane, Tg, R0);
-      load_tags<PAGED>(B, TT, min(t + 12, tlast), a, Tg);
-      if (!PAGED || !TgC1.raw) consume<PAGED, false>(R1, st, L, B, TgC1.kto, TgC1.vto, t + 4, S, A.scale_log2e, a, q, qf);
+      load_tile<PAGED>(B, t + 2 * NW, lane, Tg, R0);
+      load_tags<PAGED>(B, TT, min(t + 3 * NW, tlast), a, Tg);
+      if (!PAGED || !TgC1.raw) consume<PAGED, false>(R1, st, L, B, TgC1.kto, TgC1.vto, t + NW, S, A.scale_log2e, a, q, qf);
     }
-    const int t = t0 + 4 * i;
+    const int t = t0 + NW * i;
     if (n - i == 2) {
       TgC1 = Tg;
-      load_tile<PAGED>(B, t + 4, lane, Tg, R1);
+      load_tile<PAGED>(B, t + NW, lane, Tg, R1);
       if (!PAGED || !TgC0.raw) consume<PAGED, false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf);
-      if (!PAGED || !TgC1.raw) consume<PAGED, false>(R1, st, L, B, TgC1.kto, TgC1.vto, t + 4, S, A.scale_log2e, a, q, qf);
+      if (!PAGED || !TgC1.raw) consume<PAGED, false>(R1, st, L, B, TgC1.kto, TgC1.vto, t + NW, S, A.scale_log2e, a, q, qf);
     } else {
       if (!PAGED || !TgC0.raw) consume<PAGED, false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf);
     }
@@ -559,11 +566,11 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
   // whose K or V side is a raw tile (the block that is still filling, or escapes that did not fit the slot)
   if (PAGED) {
     bool mine = false;
-    for (int i = tid; i < thi - tlo; i += 256) mine |= (tile_table[i].x | tile_table[i].y) < 0;
+    for (int i = tid; i < thi - tlo; i += NT) mine |= (tile_table[i].x | tile_table[i].y) < 0;
     if (__syncthreads_or(mine)) {
-      RawScratch& R = *reinterpret_cast<RawScratch*>(&L.acc[0][0][0]);
-      for (int g = tid >> 7; g < G; g += 2) L.acc[4][g][tid & 127] = 0.f;
-      raw_rows_begin(R, A, qh0, G, tid);
+      RawScratch& R = *reinterpret_cast<RawScratch*>(&M.acc[0][0][0]);
+      for (int g = tid >> 7; g < G; g += NT / 128) M.acc[NW][g][tid & 127] = 0.f;
+      raw_rows_begin<NT>(R, A, qh0, G, tid);
       const uint8_t* b3k = A.k.base3 + (long)(ch % A.NB) * D; const uint8_t* b4k = A.k.base4 + (long)(ch % A.NB) * D;
       const uint8_t* b3v = A.v.base3 + (long)(ch % A.NB) * D; const uint8_t* b4v = A.v.base4 + (long)(ch % A.NB) * D;
       for (int i = 0; i < thi - tlo; ++i) {
@@ -580,16 +587,16 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
           const uint8_t* sl = A.pool + (size_t)e.y * (size_t)A.TS;
           decode_tile_rows<KIND_V>(sl, sl + SLOT_CD, reinterpret_cast<const int*>(sl + SLOT_FL), sl + SLOT_OV, b3v, b4v, lane, T, R.vrows, D);
         }
-        raw_rows_attend(R, krows, vrows, min(T, S - (tlo + i) * T), A.scale_log2e, G, tid, L.m[4], L.l[4], L.acc[4]);
+        raw_rows_attend<NT>(R, krows, vrows, min(T, S - (tlo + i) * T), A.scale_log2e, G, tid, M.m[NW], M.l[NW], M.acc[NW]);
         __syncthreads();      // staging rows are free again
       }
     }
   } else if (split == A.nsplit) {
-    RawScratch& R = *reinterpret_cast<RawScratch*>(&L.acc[0][0][0]);
+    RawScratch& R = *reinterpret_cast<RawScratch*>(&M.acc[0][0][0]);
     const int TL = slot < 0 ? 0 : min(A.tl[ch], A.tcap);
-    for (int g = tid >> 7; g < G; g += 2) L.acc[4][g][tid & 127] = 0.f;
-    raw_rows_begin(R, A, qh0, G, tid);
-    raw_rows_attend(R, A.kt + (long)ch * A.tcap * D, A.vt + (long)ch * A.tcap * D, TL, A.scale_log2e, G, tid, L.m[4], L.l[4], L.acc[4]);
+    for (int g = tid >> 7; g < G; g += NT / 128) M.acc[NW][g][tid & 127] = 0.f;
+    raw_rows_begin<NT>(R, A, qh0, G, tid);
+    raw_rows_attend<NT>(R, A.kt + (long)ch * A.tcap * D, A.vt + (long)ch * A.tcap * D, TL, A.scale_log2e, G, tid, M.m[NW], M.l[NW], M.acc[NW]);
     __syncthreads();      // the scratch view is dead before the waves publish into the same memory
   }
   // The accumulators are MFMA results: keep their first non-MFMA read a full MFMA latency away on every path.
@@ -600,30 +607,30 @@ __global__ void __launch_bounds__(256, 2) k_attn_split(const AttnArgs A) {
 
   // ---- merge the 4 waves of the block, write the split's partial
   if (a < G) {
-    if (q == 0) { L.m[wave][a] = m_run; L.l[wave][a] = l_run; }
+    if (q == 0) { M.m[wave][a] = m_run; M.l[wave][a] = l_run; }
 #pragma unroll
     for (int i = 0; i < 8; ++i)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) L.acc[wave][a][chan_v(8 * (4 * q + r) + i)] = acc[i][r];
+      for (int r = 0; r < 4; ++r) M.acc[wave][a][chan_v(8 * (4 * q + r) + i)] = acc[i][r];
   }
   __syncthreads();
   const int d = tid & 127;
-  for (int g = tid >> 7; g < G; g += 2) {
-    float M = -INFINITY;
+  for (int g = tid >> 7; g < G; g += NT / 128) {
+    float Mx = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < 5; ++w) M = fmaxf(M, L.m[w][g]);
+    for (int w = 0; w < NW + 1; ++w) Mx = fmaxf(Mx, M.m[w][g]);
     float Lc = 0.f, Ac = 0.f;
 #pragma unroll
-    for (int w = 0; w < 5; ++w) {
-      const bool live = L.m[w][g] != -INFINITY;          // an empty partial's accumulator may hold anything
-      const float f = live ? __builtin_amdgcn_exp2f(L.m[w][g] - M) : 0.f;
-      Lc += L.l[w][g] * f; Ac += live ? L.acc[w][g][d] * f : 0.f;
+    for (int w = 0; w < NW + 1; ++w) {
+      const bool live = M.m[w][g] != -INFINITY;          // an empty partial's accumulator may hold anything
+      const float f = live ? __builtin_amdgcn_exp2f(M.m[w][g] - Mx) : 0.f;
+      Lc += M.l[w][g] * f; Ac += live ? M.acc[w][g][d] * f : 0.f;
     }
     const long pidx = (qh0 + g) * A.nslot + split;
-    if (d == 0) { store_partial(A.pm + pidx, M); store_partial(A.pl + pidx, Lc); }
+    if (d == 0) { store_partial(A.pm + pidx, Mx); store_partial(A.pl + pidx, Lc); }
     store_partial(A.pa + pidx * D + d, Ac);
   }
-  publish_and_merge(A, bh, qh0, G, tid, &L.acc[0][0][0]);
+  publish_and_merge<NW>(A, bh, qh0, G, tid, &M.acc[0][0][0]);
 }
 
 // ---------------------------------------------------------------------------------------------------- split merge
@@ -798,7 +805,7 @@ __global__ void __launch_bounds__(256, 2) k_bf16_attn_split(const AttnArgs A) {
     if (d == 0) { store_partial(A.pm + pidx, M); store_partial(A.pl + pidx, Lc); }
     store_partial(A.pa + pidx * D + d, Ac);
   }
-  publish_and_merge(A, bh, qh0, G, tid, &L.acc[0][0][0]);
+  publish_and_merge<4>(A, bh, qh0, G, tid, &L.acc[0][0][0]);
 }
 
 }  // namespace gaac
@@ -828,7 +835,9 @@ static int attn_split_impl(
   A.tickets = tickets; A.out = (u16*)out;
   GAAC_REQUIRE(!tickets || out, "gaac_attn: the fused merge needs an output buffer");
   A.pool = nullptr; A.raw = nullptr; A.mt = nullptr; A.bt = nullptr; A.bt_stride = 0; A.TS = 0;
-  hipLaunchKernelGGL(k_attn_split<false>, dim3(B * n_kv, nslot), dim3(256), 0, (hipStream_t)stream, A);
+  // few blocks: one 8-wave block per CU (half as many partials); otherwise two 4-wave blocks per CU
+  if ((long)B * n_kv * nslot <= 256) hipLaunchKernelGGL((k_attn_split<false, 8>), dim3(B * n_kv, nslot), dim3(512), 0, (hipStream_t)stream, A);
+  else hipLaunchKernelGGL((k_attn_split<false, 4>), dim3(B * n_kv, nslot), dim3(256), 0, (hipStream_t)stream, A);
   return launch_status("gaac_attn(split)");
 }
 
@@ -892,7 +901,8 @@ extern "C" int gaac_paged_attn(
   A.kt = nullptr; A.vt = nullptr; A.tl = nullptr; A.tcap = 0;
   A.tickets = tickets; A.out = (u16*)out;
   A.pool = pool; A.raw = (const u16*)raw; A.mt = mt; A.bt = bt; A.bt_stride = bt_stride; A.TS = TS;
-  hipLaunchKernelGGL(k_attn_split<true>, dim3(B * n_kv, nsplit), dim3(256), 0, (hipStream_t)stream, A);
+  if ((long)B * n_kv * nsplit <= 256) hipLaunchKernelGGL((k_attn_split<true, 8>), dim3(B * n_kv, nsplit), dim3(512), 0, (hipStream_t)stream, A);
+  else hipLaunchKernelGGL((k_attn_split<true, 4>), dim3(B * n_kv, nsplit), dim3(256), 0, (hipStream_t)stream, A);
   return launch_status("gaac_paged_attn");
 }
 

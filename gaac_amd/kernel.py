@@ -18,15 +18,16 @@ def _ext():
     return _lib.load()
 
 
-def choose_nsplit(B: int, n_kv: int, S: int, target_ctas: int = 512, min_tok: int = 256, cap: int = 256) -> int:
-    """Splits per (row, kv head): about 2 four-wave blocks per CU of the 256-CU MI355X (the reference targets 96 CTAs
-    for a 48-SM part, kernel.py:340-342), at least min_tok tokens per split."""
+def choose_nsplit(B: int, n_kv: int, S: int, target_ctas: int = 256, min_tok: int = 256, cap: int = 256) -> int:
+    """Splits per (row, kv head): one eight-wave block per CU of the 256-CU MI355X (the reference targets 96 CTAs for a 48-SM
+    part, kernel.py:340-342), at least min_tok tokens per split.  Launches of up to 256 blocks use eight-wave blocks, larger
+    ones four-wave blocks (two per CU)."""
     return min(max(1, target_ctas // (B * n_kv)), max(1, S // min_tok), cap)
 
 
-def nsplit_with_tail_row(nsplit: int, B: int, n_kv: int, resident: int = 512) -> int:
+def nsplit_with_tail_row(nsplit: int, B: int, n_kv: int, resident: int = 256) -> int:
     """The raw tail adds one block row to the launch: give up one split when that row would no longer be resident together with the
-    others (2 blocks on each of the 256 CUs), so that no block has to wait for a free CU."""
+    others (one eight-wave block on each of the 256 CUs), so that no block has to wait for a free CU."""
     return nsplit - 1 if nsplit > 1 and B * n_kv * nsplit <= resident < B * n_kv * (nsplit + 1) else nsplit
 
 

@@ -17,9 +17,10 @@ SM_OFF, CD_OFF, FL_OFF, OVF_OFF = 0, 2048, 2816, 2880   # byte layout of a tile 
 MAX_TILES_PER_SPLIT = 1024
 
 
-def choose_nsplit(B: int, n_kv: int, S: int, target_ctas: int = 512, min_tok: int = 256, cap: int = 256) -> int:
-    """Splits per (row, kv head): about two blocks per CU, at least min_tok tokens each, and never more than 1024 tiles per split
-    (the kernel keeps one split's slot lookups in LDS)."""
+def choose_nsplit(B: int, n_kv: int, S: int, target_ctas: int = 2048, min_tok: int = 256, cap: int = 256) -> int:
+    """Splits per (row, kv head) for the longest sequence S of the batch: sequences of a serving batch differ in length, so the
+    launch is cut into several times more blocks than the 512 that are resident (they balance out as they are scheduled), at
+    least min_tok tokens each, and never more than 1024 tiles per split (the kernel keeps one split's slot lookups in LDS)."""
     need = -(-(-(-S // BLOCK)) // MAX_TILES_PER_SPLIT)
     return max(min(max(1, target_ctas // (B * n_kv)), max(1, S // min_tok), cap), need, 1)
 

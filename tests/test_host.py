@@ -82,7 +82,7 @@ def test_storage_index_is_a_bijection_and_perms_match_closed_forms():
 
 def test_choose_nsplit_bounds():
     from gaac_amd.kernel import choose_nsplit
-    assert choose_nsplit(1, 8, 65536) == 64            # 512 blocks over 8 kv heads
+    assert choose_nsplit(1, 8, 65536) == 32            # 256 blocks over 8 kv heads
     assert choose_nsplit(1, 8, 300) == 1               # never below 256 tokens per split
     assert choose_nsplit(64, 8, 65536) == 1
     assert choose_nsplit(1, 1, 1 << 20) == 256         # cap
