@@ -733,7 +733,7 @@ __global__ void __launch_bounds__(256, 2) k_bf16_attn_split(const AttnArgs A) {
   const int bh = blockIdx.x, split = blockIdx.y, tid = threadIdx.x;
   const int b = bh / A.n_kv, kvh = bh % A.n_kv, G = A.G;
   const long qh0 = (long)b * A.n_q + (long)kvh * G;
-  const int S = A.tcap;
+  const int S = A.sl ? min(max(A.sl[b], 0), A.tcap) : A.tcap;      // per-row lengths on the device (decode steps inside a graph) or one length
   const int ntiles = (S + T - 1) / T, chunk = (ntiles + A.nsplit - 1) / A.nsplit;
   const int tlo = min(split * chunk, ntiles), thi = min(tlo + chunk, ntiles);
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, a = lane & 15, q = lane >> 4;
@@ -906,8 +906,8 @@ extern "C" int gaac_paged_attn(
   return launch_status("gaac_paged_attn");
 }
 
-extern "C" int gaac_bf16_attn(const void* k, const void* v, int S, long head_stride_tokens, const void* q, int B, int n_q, int n_kv,
-                              float scale, int nsplit, float* pm, float* pl, float* pa, int* tickets, void* out, void* stream) {
+extern "C" int gaac_bf16_attn(const void* k, const void* v, int S, const int* seq_lens, long head_stride_tokens, const void* q, int B, int n_q,
+                              int n_kv, float scale, int nsplit, float* pm, float* pl, float* pa, int* tickets, void* out, void* stream) {
   GAAC_REQUIRE(n_kv > 0 && n_q > 0 && n_q % n_kv == 0 && n_q / n_kv <= GMAX, "GQA group size must be 1..%d (n_q=%d, n_kv=%d)", GMAX, n_q, n_kv);
   GAAC_REQUIRE(k && v && q && pm && pl && pa && tickets && out, "gaac_bf16_attn: null pointer");
   GAAC_REQUIRE(B > 0 && S > 0 && head_stride_tokens >= S && nsplit >= 1 && nsplit <= MAX_SLOTS, "gaac_bf16_attn: bad sizes");
@@ -915,7 +915,7 @@ extern "C" int gaac_bf16_attn(const void* k, const void* v, int S, long head_str
   A.q = (const u16*)q; A.pm = pm; A.pl = pl; A.pa = pa;
   A.S_pad = (int)head_stride_tokens; A.scale_log2e = scale * 1.4426950408889634f; A.nsplit = nsplit; A.nslot = nsplit;
   A.n_kv = n_kv; A.n_q = n_q; A.G = n_q / n_kv; A.NB = 1;
-  A.kt = (const u16*)k; A.vt = (const u16*)v; A.tcap = S;
+  A.kt = (const u16*)k; A.vt = (const u16*)v; A.tcap = S; A.sl = seq_lens;
   A.tickets = tickets; A.out = (u16*)out;
   hipLaunchKernelGGL(k_bf16_attn_split, dim3(B * n_kv, nsplit), dim3(256), 0, (hipStream_t)stream, A);
   return launch_status("gaac_bf16_attn");

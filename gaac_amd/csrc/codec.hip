@@ -79,29 +79,36 @@ __global__ void __launch_bounds__(64) k_compact(const uint8_t* __restrict__ esc_
   for (int k = threadIdx.x; k < n; k += 64) dst[k] = src[k];
 }
 
+// One block per (head, chunk of 2048 tag words): the bytes of all earlier chunks are re-summed by the block itself (a few hundred KB
+// out of L2 at most), then the chunk is scanned: 8 words per thread serially, thread totals by a block scan.
+constexpr int RO_CHUNK = 2048;
 __global__ void __launch_bounds__(256) k_row_offsets(const int* __restrict__ flags, int S, int S_pad, int* __restrict__ out) {
   __shared__ int sh[256];
-  __shared__ int carry;
-  const int h = blockIdx.x, tid = threadIdx.x;
-  if (tid == 0) carry = 0;
+  const int h = blockIdx.y, c = blockIdx.x, tid = threadIdx.x;
+  const int* f = flags + (long)h * S_pad;
+  int before = 0;
+  for (int s = tid; s < c * RO_CHUNK; s += 256) before += esc_bytes((u32)f[s]);
+  const int s0 = c * RO_CHUNK + tid * 8;
+  int rb[8], mine = 0;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) { rb[k] = s0 + k < S ? esc_bytes((u32)f[s0 + k]) : 0; mine += rb[k]; }
+  // block-wide: sum of `before`, inclusive scan of `mine`
+  sh[tid] = before;
   __syncthreads();
-  for (int base = 0; base < S; base += 256) {
-    const int s = base + tid;
-    const int rb = s < S ? esc_bytes((u32)flags[(long)h * S_pad + s]) : 0;
-    sh[tid] = rb;
+  for (int o = 128; o > 0; o >>= 1) { if (tid < o) sh[tid] += sh[tid + o]; __syncthreads(); }
+  const int base = sh[0];
+  __syncthreads();
+  sh[tid] = mine;
+  __syncthreads();
+  for (int o = 1; o < 256; o <<= 1) {
+    const int v = tid >= o ? sh[tid - o] : 0;
     __syncthreads();
-    for (int o = 1; o < 256; o <<= 1) {
-      int v = tid >= o ? sh[tid - o] : 0;
-      __syncthreads();
-      sh[tid] += v;
-      __syncthreads();
-    }
-    const int c = carry;
-    if (s < S) out[(long)h * S + s] = c + sh[tid] - rb;
-    __syncthreads();
-    if (tid == 255) carry = c + sh[255];
+    sh[tid] += v;
     __syncthreads();
   }
+  int off = base + sh[tid] - mine;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) { if (s0 + k < S) out[(long)h * S + s0 + k] = off; off += rb[k]; }
 }
 
 // ---------------------------------------------------------------------------------------------------- page decoder
@@ -173,7 +180,7 @@ int gaac_compact(const uint8_t* esc_slots, const int* tile_bytes, const int* til
 
 int gaac_row_offsets(const int* flags, int H, int S, int S_pad, int* out, void* stream) {
   GAAC_REQUIRE(flags && out && H > 0 && S > 0 && S_pad >= S, "gaac_row_offsets: bad arguments");
-  hipLaunchKernelGGL(k_row_offsets, dim3(H), dim3(256), 0, (hipStream_t)stream, flags, S, S_pad, out);
+  hipLaunchKernelGGL(k_row_offsets, dim3((S + RO_CHUNK - 1) / RO_CHUNK, H), dim3(256), 0, (hipStream_t)stream, flags, S, S_pad, out);
   return launch_status("gaac_row_offsets");
 }
 

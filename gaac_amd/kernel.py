@@ -96,15 +96,18 @@ def attention(q, kp, vp, scale=None, nsplit=None, phase="fused"):
     return out.view(B, n_q, Dq)
 
 
-def bf16_attention(q, k, v, scale=None, nsplit=None, ws=None):
-    """Baseline: decode attention over UNCOMPRESSED K/V (k, v: [B*n_kv, S, D] bf16 contiguous; q: [B, n_q, D]) with the kernel
-    structure of the compressed path minus the decoder.  Returns [B, n_q, D] bf16."""
+def bf16_attention(q, k, v, scale=None, nsplit=None, ws=None, seq_lens=None, out=None):
+    """Baseline: decode attention over UNCOMPRESSED K/V (k, v: [B*n_kv, S, D] bf16, rows contiguous; q: [B, n_q, D]) with the kernel
+    structure of the compressed path minus the decoder.  seq_lens: optional int32 [B] device tensor of valid tokens per batch row
+    (<= S).  Returns [B, n_q, D] bf16."""
     B, n_q, Dq = q.shape
     H, S, _ = k.shape
     n_kv = H // B
+    if k.stride(1) != D or v.stride(1) != D or k.stride(0) != v.stride(0): raise RuntimeError("bf16_attention expects token rows of 128 contiguous elements")
     if nsplit is None: nsplit = choose_nsplit(B, n_kv, S)
-    if ws is None: ws = AttnWorkspace(B * n_q, nsplit, q.dtype, q.device)
+    if ws is None: ws = AttnWorkspace(B * n_q, nsplit, q.dtype, q.device, with_out=out is None)
+    if out is None: out = ws.out if ws.out is not None else torch.empty(B * n_q, D, dtype=q.dtype, device=q.device)
     p = _lib.ptr
-    _lib.call("gaac_bf16_attn", p(k), p(v), S, k.stride(0) // D, p(q.contiguous()), B, n_q, n_kv, float(scale if scale is not None else Dq ** -0.5),
-              nsplit, p(ws.pm), p(ws.pl), p(ws.pa), p(ws.tickets), p(ws.out), _lib.stream())
-    return ws.out.view(B, n_q, Dq)
+    _lib.call("gaac_bf16_attn", p(k), p(v), S, p(seq_lens), k.stride(0) // D, p(q.contiguous()), B, n_q, n_kv,
+              float(scale if scale is not None else Dq ** -0.5), nsplit, p(ws.pm), p(ws.pl), p(ws.pa), p(ws.tickets), p(out), _lib.stream())
+    return out.view(B, n_q, Dq)

@@ -125,10 +125,11 @@ int gaac_paged_attn(const uint8_t* pool, int TS, const void* raw, const int* mt,
                     float* pm, float* pl, float* pa, int* tickets, void* out, void* stream);
 
 /* Baseline, not part of the compressed path: decode attention over UNCOMPRESSED bf16 K/V [B*n_kv][head_stride_tokens][128] (S tokens
- * per head) with the same block / wave / MFMA structure, merge and partial buffers as gaac_attn_fused.  The reference compares
- * against flash-attn (examples/attention.py:29-30); this is the same-GPU counterpart for that comparison. */
-int gaac_bf16_attn(const void* k, const void* v, int S, long head_stride_tokens, const void* q, int B, int n_q, int n_kv,
-                   float scale, int nsplit, float* pm, float* pl, float* pa, int* tickets, void* out, void* stream);
+ * per head, or seq_lens[b] <= S tokens for batch row b when seq_lens != NULL) with the same block / wave / MFMA structure, merge and
+ * partial buffers as gaac_attn_fused.  The reference compares against flash-attn (examples/attention.py:29-30); this is the same-GPU
+ * counterpart for that comparison. */
+int gaac_bf16_attn(const void* k, const void* v, int S, const int* seq_lens, long head_stride_tokens, const void* q, int B, int n_q,
+                   int n_kv, float scale, int nsplit, float* pm, float* pl, float* pa, int* tickets, void* out, void* stream);
 
 /* Measurement aid with no counterpart in the reference: a plain copy of nbytes (multiple of 16) with 16-byte accesses per lane,
  * the known-size kernel that HBM traffic counters (FETCH_SIZE / WRITE_SIZE) are scaled against. */
