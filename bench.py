@@ -81,9 +81,10 @@ def main():
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="also run the library's plain 64 MiB copy kernel 10 times (the known-size kernel for scaling FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--cpu-heads", type=int, default=8, help="kv heads in the CPU baseline sample (0 = skip)")
-    ap.add_argument("--workload", default="decode64k", choices=["decode64k", "decode64k_g6", "codec", "paged", "serve"],
+    ap.add_argument("--workload", default="decode64k", choices=["decode64k", "decode64k_g6", "codec", "paged", "serve", "phases"],
                     help="decode64k = the headline (config 1); decode64k_g6 = config 2 (24 q / 4 kv heads, V sigma in 2^[-2,2]); "
-                         "codec = config 0 round trip; paged = config 3 serving step; serve = config 4 end-to-end decode")
+                         "codec = config 0 round trip; paged = config 3 serving step; serve = config 4 end-to-end decode; "
+                         "phases = per-block phase time stamps of the config 1 kernel (instrumented build)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one MI355X; this build has no multi-GPU path (the hot path shards by kv head without any exchange). Use --gpus 1.", file=sys.stderr)
@@ -96,6 +97,7 @@ def main():
     if a.workload == "codec": return bench_codec(a)
     if a.workload == "paged": return bench_paged(a)
     if a.workload == "serve": return bench_serve(a)
+    if a.workload == "phases": return bench_phases(a)
     from gaac_amd import Codec, TileEncoder
     from gaac_amd.kernel import attn_launch, choose_nsplit, nsplit_with_tail_row, AttnWorkspace
     dev = "cuda"
@@ -377,6 +379,54 @@ def bench_serve(a):
     res["same_tokens_fraction"] = round((toks["gaac"] == toks["bf16"]).float().mean().item(), 4)
     res["speedup"] = round(res["gaac"]["tokens_per_s"] / res["bf16"]["tokens_per_s"], 4)
     print(json.dumps(res))
+
+
+def bench_phases(a):
+    """Where a launch of the config 1 kernel spends its time: the instrumented build (libgaac_hip_timing.so) stamps the 100 MHz wall
+    clock per block at entry, after the first loads, at table readiness, at each wave's loop end, after the partial stores and at exit."""
+    import ctypes
+    from gaac_amd import build as gbuild
+    if not os.path.exists(gbuild.LIB_TIMING):
+        print("build the instrumented library first: python -m gaac_amd.build", file=sys.stderr); sys.exit(2)
+    os.environ["GAAC_HIP_LIB"] = gbuild.LIB_TIMING
+    from gaac_amd import Codec, TileEncoder, _lib
+    from gaac_amd.kernel import attn_launch, choose_nsplit, nsplit_with_tail_row, AttnWorkspace
+    dev = "cuda"
+    n_q, H = N_KV * G, N_KV
+    kd, vd = make_kv(1, H, S_CTX + TAIL_TOK).to(dev), make_kv(2, H, S_CTX + TAIL_TOK).to(dev)
+    ck, cv = Codec(N_KV).calibrate(kd[:, :1024]), Codec(N_KV).calibrate(vd[:, :1024])
+    kp = TileEncoder("k").encode(ck, kd[:, :S_CTX].contiguous()); vp = TileEncoder("v").encode(cv, vd[:, :S_CTX].contiguous())
+    pages = [(kp, vp)] + [(clone_store(kp), clone_store(vp)) for _ in range(a.copies - 1)]
+    kt = torch.zeros(H, 16, D, dtype=torch.bfloat16, device=dev); vt = torch.zeros_like(kt)
+    kt[:, :TAIL_TOK] = kd[:, S_CTX:]; vt[:, :TAIL_TOK] = vd[:, S_CTX:]
+    TL = torch.full((H,), TAIL_TOK, dtype=torch.int32, device=dev); SL = torch.full((H,), S_CTX, dtype=torch.int32, device=dev)
+    slots = torch.zeros(1, dtype=torch.int32, device=dev)
+    q2d = torch.randn(n_q, D, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16).to(dev)
+    nsplit = a.nsplit or nsplit_with_tail_row(choose_nsplit(1, N_KV, S_CTX), 1, N_KV)
+    nblk = H * (nsplit + 1)
+    NW = 8 if nblk <= 256 else 4
+    ws = AttnWorkspace(n_q, nsplit + 1, torch.bfloat16, dev)
+    dbg = torch.zeros(nblk * 16, dtype=torch.int64, device=dev)
+    lib = _lib.load(); lib.gaac_set_phase_buffer.argtypes = [ctypes.c_void_p]; lib.gaac_set_phase_buffer.restype = None
+    lib.gaac_set_phase_buffer(dbg.data_ptr())
+    f = lambda i: attn_launch(pages[i % len(pages)][0], pages[i % len(pages)][1], q2d, slots, n_q, N_KV, SL, S_CTX, D ** -0.5, nsplit, kt, vt, TL, 16, ws=ws)
+    for i in range(10): f(i)
+    rows = []
+    for i in range(20):
+        dbg.zero_(); torch.cuda.synchronize(); f(i); torch.cuda.synchronize()
+        raw = dbg.cpu().numpy().astype(np.float64) * 0.01          # us
+        t = raw[:nblk * 8].reshape(nblk, 8); t0 = t[:, 0].min()
+        main = t[H:] - t0                                            # blocks after the tail blocks
+        wv = raw[nblk * 8:].reshape(nblk, 8)[H:, :NW] - t0
+        xcd = (np.arange(nblk - H) + H) % 8
+        ends = wv.max(1)
+        rows.append([main[:, 0].max(), main[:, 6].mean(), main[:, 1].mean(), wv[:, :4].mean(), wv[:, NW - 4:].mean(), ends.mean(), ends.max(),
+                     main[:, 4].mean(), main[:, 4].max(), (t[:, 5] - t0).max(), min(ends[xcd == x].mean() for x in range(8)), max(ends[xcd == x].mean() for x in range(8))])
+    m = np.median(np.array(rows), 0)
+    names = ["last_block_start", "first_tile_loads_issued_mean", "tables_ready_mean", "loop_end_waves_0_3_mean", f"loop_end_waves_{NW - 4}_{NW - 1}_mean",
+             "block_loop_end_mean", "block_loop_end_max", "partial_stored_mean", "partial_stored_max", "last_stamp", "loop_end_fastest_xcd_mean", "loop_end_slowest_xcd_mean"]
+    print(json.dumps({"workload": "config 1 kernel phases, us from the first block's entry (median of 20 launches, each after a device synchronize)",
+                      "nsplit": nsplit, "waves_per_block": NW, **{k: round(float(v), 2) for k, v in zip(names, m)}}))
 
 
 if __name__ == "__main__":

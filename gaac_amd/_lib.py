@@ -33,17 +33,19 @@ _SIGNATURES = {
 
 
 def lib_path() -> str:
-    return _LIB_PATH
+    """The library file: gaac_amd/libgaac_hip.so, or the instrumented build named by GAAC_HIP_LIB (read when the library is loaded)."""
+    return os.environ.get("GAAC_HIP_LIB") or _LIB_PATH
 
 
 def load():
     """The loaded library (ctypes.CDLL).  Raises if it has not been built (python -m gaac_amd.build)."""
     global _lib
     if _lib is None:
-        if not os.path.exists(_LIB_PATH):
-            raise RuntimeError(f"{_LIB_PATH} is missing: build it with `python -m gaac_amd.build` (hipcc, gfx950). "
+        path = lib_path()
+        if not os.path.exists(path):
+            raise RuntimeError(f"{path} is missing: build it with `python -m gaac_amd.build` (hipcc, gfx950). "
                                "gaac_amd has no CPU or PyTorch fallback.")
-        lib = ctypes.CDLL(_LIB_PATH)
+        lib = ctypes.CDLL(path)
         lib.gaac_last_error.restype = ctypes.c_char_p
         lib.gaac_last_error.argtypes = []
         for name, args in _SIGNATURES.items():

@@ -9,17 +9,20 @@ import os, subprocess, sys, shutil
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libgaac_hip.so")
+LIB_TIMING = os.path.join(HERE, "libgaac_hip_timing.so")      # same sources with -DGAAC_PHASE_TIMING (per-block phase time stamps)
 SOURCES = ["codec.hip", "attn.hip", "cache.hip", "paged.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", 
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",      # never emit packed-FP32 VALU ops
          "-Wno-unused-command-line-argument"]
 
 
-def build(verbose: bool = True, extra_flags: list[str] | None = None) -> str:
+def build(verbose: bool = True, extra_flags: list[str] | None = None, timing: bool = False) -> str:
+    """timing=True builds the instrumented variant (libgaac_hip_timing.so, loaded through the GAAC_HIP_LIB override)."""
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     objs = []
+    if timing: extra_flags = [*(extra_flags or []), "-DGAAC_PHASE_TIMING"]
     for src in SOURCES:
-        obj = os.path.join(CSRC, src.replace(".hip", ".o"))
+        obj = os.path.join(CSRC, src.replace(".hip", ".timing.o" if timing else ".o"))
         cmd = [hipcc, *FLAGS, *(extra_flags or []), "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose: print(" ".join(cmd), flush=True)
         r = subprocess.run(cmd, capture_output=True, text=True)
@@ -28,13 +31,15 @@ def build(verbose: bool = True, extra_flags: list[str] | None = None) -> str:
             raise RuntimeError(f"hipcc failed on {src}:\n{err}")
         if verbose and err.strip(): print(err, file=sys.stderr)
         objs.append(obj)
-    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", LIB]
+    out = LIB_TIMING if timing else LIB
+    cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", out]
     if verbose: print(" ".join(cmd), flush=True)
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError(f"link failed:\n{r.stderr}")
-    return LIB
+    return out
 
 
 if __name__ == "__main__":
     print(build())
+    print(build(timing=True))

@@ -34,7 +34,15 @@ struct AttnArgs {
   // paged slot pool (k_attn_split<true>): sl = tokens per batch row, bt = block table [B][bt_stride], mt = mode table, pool = tile
   // slots of TS bytes, raw = side pool of BF16 tiles; physical tile = block*2*n_kv + 2*kvh + kind
   const uint8_t* pool; const u16* raw; const int* mt; const int* bt; int bt_stride; int TS;
+#ifdef GAAC_PHASE_TIMING
+  long long* dbg;
+#endif
 };
+#ifdef GAAC_PHASE_TIMING
+#define GAAC_STAMP(k) do { if (A.dbg && threadIdx.x == 0) A.dbg[(long)blockIdx.x * 8 + (k)] = wall_clock64(); } while (0)
+#else
+#define GAAC_STAMP(k) do {} while (0)
+#endif
 constexpr int MAX_CHUNK = 1024;  // tiles per split whose slot lookups a block keeps in LDS (paged mode)
 constexpr int SLOT_CD = TILE_SM, SLOT_FL = TILE_SM + TILE_CD, SLOT_OV = SLOT_FL + 4 * T;      // byte offsets inside a tile slot
 
@@ -463,6 +471,13 @@ __device__ __forceinline__ void consume(const TileRegs& R, WaveState& st, const 
     consume_tile<PAGED, PARTIAL, false>(R, st, L, B, kto, vto, tile, S, scale_log2e, a, q, qf);
 }
 
+// next tile index from the block's counter (one LDS atomic per wave, the result is uniform)
+__device__ __forceinline__ int take_tile(int* ctr, int lane) {
+  int v = 0;
+  if (lane == 0) v = atomicAdd(ctr, 1);
+  return __builtin_amdgcn_readfirstlane(v);
+}
+
 // ---------------------------------------------------------------------------------------------------- main kernel
 // NW = waves per block: 4 (two blocks per CU) or 8 (one block per CU: half as many partials to merge for the same occupancy)
 template <bool PAGED, int NW>
@@ -471,10 +486,15 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
   __shared__ AttnLds L;
   __shared__ MergeLds<NW> M;
   __shared__ int2 tile_table[PAGED ? MAX_CHUNK : 1];
-  const int bh = blockIdx.x, tid = threadIdx.x;
-  // with a raw tail the grid has one more block row: it is dispatched first (blockIdx.y == 0), owns no compressed tile and writes
-  // partial slot nsplit
-  const int split = A.nslot > A.nsplit ? (blockIdx.y == 0 ? A.nsplit : (int)blockIdx.y - 1) : (int)blockIdx.y;
+  __shared__ int next_tile;
+  const int tid = threadIdx.x;
+  GAAC_STAMP(0);
+  // One-dimensional grid.  With a raw tail there is one more block per (row, kv head): those are dispatched first, own no compressed
+  // tile and write partial slot nsplit.  The other blocks are numbered split-fastest, so the splits of one kv head go round the
+  // eight XCDs (workgroups are dealt to XCDs in turn) instead of all landing on one: heads with heavier tiles then load every XCD alike.
+  const int n_bh = (int)gridDim.x / A.nslot, n_tail = A.nslot > A.nsplit ? n_bh : 0;
+  const int lin = (int)blockIdx.x - n_tail;
+  const int bh = lin < 0 ? (int)blockIdx.x : lin / A.nsplit, split = lin < 0 ? A.nsplit : lin % A.nsplit;
   const int b = bh / A.n_kv, kvh = bh % A.n_kv, G = A.G;
   const int slot = PAGED ? 0 : A.slot[b], ch = PAGED ? kvh : (slot < 0 ? 0 : slot) * A.n_kv + kvh;
   const long qh0 = (long)b * A.n_q + (long)kvh * G;
@@ -503,25 +523,30 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
     B.TS = 0;
   }
 
-  // tiles of this wave: t(i) = tlo + wave + NW i, i < n.  Ping-pong registers R0/R1; tag words are fetched one tile further
-  // ahead (index clamped to the wave's last tile, so that no load sits under a branch the consumer has to join).  A partly
-  // filled last tile of the sequence is taken out of the pipeline and handled at the end by the wave that owns it.
-  const int t0 = tlo + wave;
-  const int n_all = t0 < thi ? (thi - t0 + NW - 1) / NW : 0;
-  const bool own_partial = n_all > 0 && (S % T) != 0 && t0 + NW * (n_all - 1) == ntiles - 1;
-  const int n = n_all - (own_partial ? 1 : 0);
-  const int tlast = t0 + NW * (n - 1);
+  // Tiles are handed out dynamically: each wave starts with tiles tlo + wave and tlo + NW + wave and takes every further one from
+  // a counter in LDS.  Of the two waves that share a SIMD the older one wins the issue arbitration and runs ahead; with a static
+  // split it would finish long before the other, which then runs alone and cannot hide its own latencies.  Ping-pong registers
+  // R0/R1; tag words are fetched one tile further ahead; indices past the end are clamped for the loads (no load sits under a
+  // branch the consumer has to join) and not consumed.  A partly filled last tile of the sequence is handled at the end by wave 0.
+  const bool part_here = (S % T) != 0 && thi == ntiles && thi > tlo;
+  const int thd = thi - (part_here ? 1 : 0);
+  const int tcl = max(thd - 1, tlo);
+  int tA = tlo + wave, tB = tA + NW;
   TileRegs R0, R1;
   TagRegs Tg, TgC0, TgC1;
-  if (n > 0) {          // start the first tile's loads before waiting for the block tables
-    load_tags<PAGED>(B, TT, t0, a, Tg);
+  if (tA < thd) {          // start the first tile's loads before waiting for the block tables
+    load_tags<PAGED>(B, TT, tA, a, Tg);
     TgC0 = Tg;
-    load_tile<PAGED>(B, t0, lane, Tg, R0);
-    load_tags<PAGED>(B, TT, min(t0 + NW, tlast), a, Tg);
+    load_tile<PAGED>(B, tA, lane, Tg, R0);
+    load_tags<PAGED>(B, TT, min(tB, tcl), a, Tg);
   }
+  if (tid == 0) next_tile = tlo + 2 * NW;
+  GAAC_STAMP(6);
   if (tid < 256) tables_store(L, Tr, tid);
+  GAAC_STAMP(7);
   if (tid < GMAX) { M.m[NW][tid] = -INFINITY; M.l[NW][tid] = 0.f; }
   __syncthreads();        // block tables are ready
+  GAAC_STAMP(1);
   // Q as the B operand of the score product: lane (head a, quad q), product u covers group 4q+u in word order (e, e+4);
   // exponent-base words of the lane's units
   u32x4 qf[4];
@@ -533,30 +558,29 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
   for (int i = 0; i < 8; ++i) st.acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   st.m_run = -INFINITY; st.mu_run = 0.f; st.l_run = 0.f;
 
-  if (n > 0) {
-    int i = 0;
-    for (; i + 2 < n; i += 2) {
-      const int t = t0 + NW * i;
+  if (tA < thd) {
+    int tC = take_tile(&next_tile, lane);
+    while (true) {        // R0 = tile tA, Tg = tags of tile tB
       TgC1 = Tg;
-      load_tile<PAGED>(B, t + NW, lane, Tg, R1);
-      load_tags<PAGED>(B, TT, min(t + 2 * NW, tlast), a, Tg);
-      if (!PAGED || !TgC0.raw) consume<PAGED, false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf);
+      load_tile<PAGED>(B, min(tB, tcl), lane, Tg, R1);
+      const int tD = take_tile(&next_tile, lane);
+      load_tags<PAGED>(B, TT, min(tC, tcl), a, Tg);
+      if (!PAGED || !TgC0.raw) consume<PAGED, false>(R0, st, L, B, TgC0.kto, TgC0.vto, tA, S, A.scale_log2e, a, q, qf);
+      if (tB >= thd) break;
       TgC0 = Tg;
-      load_tile<PAGED>(B, t + 2 * NW, lane, Tg, R0);
-      load_tags<PAGED>(B, TT, min(t + 3 * NW, tlast), a, Tg);
-      if (!PAGED || !TgC1.raw) consume<PAGED, false>(R1, st, L, B, TgC1.kto, TgC1.vto, t + NW, S, A.scale_log2e, a, q, qf);
-    }
-    const int t = t0 + NW * i;
-    if (n - i == 2) {
-      TgC1 = Tg;
-      load_tile<PAGED>(B, t + NW, lane, Tg, R1);
-      if (!PAGED || !TgC0.raw) consume<PAGED, false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf);
-      if (!PAGED || !TgC1.raw) consume<PAGED, false>(R1, st, L, B, TgC1.kto, TgC1.vto, t + NW, S, A.scale_log2e, a, q, qf);
-    } else {
-      if (!PAGED || !TgC0.raw) consume<PAGED, false>(R0, st, L, B, TgC0.kto, TgC0.vto, t, S, A.scale_log2e, a, q, qf);
+      load_tile<PAGED>(B, min(tC, tcl), lane, Tg, R0);
+      const int tE = take_tile(&next_tile, lane);
+      load_tags<PAGED>(B, TT, min(tD, tcl), a, Tg);
+      if (!PAGED || !TgC1.raw) consume<PAGED, false>(R1, st, L, B, TgC1.kto, TgC1.vto, tB, S, A.scale_log2e, a, q, qf);
+      if (tC >= thd) break;
+      tA = tC; tB = tD; tC = tE;
     }
   }
-  if (own_partial) {
+  GAAC_STAMP(2);
+#ifdef GAAC_PHASE_TIMING
+  if (A.dbg && lane == 0) A.dbg[((long)gridDim.x + blockIdx.x) * 8 + wave] = wall_clock64();
+#endif
+  if (part_here && wave == 0) {
     const int t = ntiles - 1;
     load_tags<PAGED>(B, TT, t, a, Tg);
     load_tile<PAGED>(B, t, lane, Tg, R0);
@@ -601,6 +625,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
   }
   // The accumulators are MFMA results: keep their first non-MFMA read a full MFMA latency away on every path.
   asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");
+  GAAC_STAMP(3);
   float l_run = quad_rows_sum(st.l_run);
   const float m_run = st.m_run == -INFINITY ? -INFINITY : st.mu_run;     // partial maxima are stored in the base-2 domain
   f32x4 (&acc)[8] = st.acc;
@@ -630,7 +655,9 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
     if (d == 0) { store_partial(A.pm + pidx, Mx); store_partial(A.pl + pidx, Lc); }
     store_partial(A.pa + pidx * D + d, Ac);
   }
+  GAAC_STAMP(4);
   publish_and_merge<NW>(A, bh, qh0, G, tid, &M.acc[0][0][0]);
+  GAAC_STAMP(5);
 }
 
 // ---------------------------------------------------------------------------------------------------- split merge
@@ -738,12 +765,14 @@ __global__ void __launch_bounds__(256, 2) k_bf16_attn_split(const AttnArgs A) {
   const int tlo = min(split * chunk, ntiles), thi = min(tlo + chunk, ntiles);
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, a = lane & 15, q = lane >> 4;
   const u16* kh = A.kt + (long)bh * A.S_pad * D; const u16* vh = A.vt + (long)bh * A.S_pad * D;
-  const int t0 = tlo + wave;
-  const int n_all = t0 < thi ? (thi - t0 + 3) / 4 : 0;
-  const bool own_partial = n_all > 0 && (S % T) != 0 && t0 + 4 * (n_all - 1) == ntiles - 1;
-  const int n = n_all - (own_partial ? 1 : 0);
+  // dynamic tile hand-out as in k_attn_split
+  __shared__ int next_tile;
+  const bool part_here = (S % T) != 0 && thi == ntiles && thi > tlo;
+  const int thd = thi - (part_here ? 1 : 0), tcl = max(thd - 1, tlo);
+  int tA = tlo + wave, tB = tA + 4;
   RawTile R0, R1;
-  if (n > 0) load_raw_tile(kh, vh, t0, S, a, q, R0);
+  if (tA < thd) load_raw_tile(kh, vh, tA, S, a, q, R0);
+  if (tid == 0) next_tile = tlo + 8;
   // Q as the B operand: lane (head a, quad q), product j covers channels 32 j + 8 q .. + 8 (rows >= G are zero)
   for (int i = tid; i < GMAX * NG; i += 256) {
     const int h = i >> 4, c = i & 15;
@@ -757,25 +786,20 @@ __global__ void __launch_bounds__(256, 2) k_bf16_attn_split(const AttnArgs A) {
 #pragma unroll
   for (int i = 0; i < 8; ++i) st.acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   st.m_run = -INFINITY; st.mu_run = 0.f; st.l_run = 0.f;
-  if (n > 0) {
-    int i = 0;
-    for (; i + 2 < n; i += 2) {
-      const int t = t0 + 4 * i;
-      load_raw_tile(kh, vh, t + 4, S, a, q, R1);
-      consume_raw_tile<false>(R0, st, t, S, A.scale_log2e, q, qf);
-      load_raw_tile(kh, vh, t + 8, S, a, q, R0);
-      consume_raw_tile<false>(R1, st, t + 4, S, A.scale_log2e, q, qf);
-    }
-    const int t = t0 + 4 * i;
-    if (n - i == 2) {
-      load_raw_tile(kh, vh, t + 4, S, a, q, R1);
-      consume_raw_tile<false>(R0, st, t, S, A.scale_log2e, q, qf);
-      consume_raw_tile<false>(R1, st, t + 4, S, A.scale_log2e, q, qf);
-    } else {
-      consume_raw_tile<false>(R0, st, t, S, A.scale_log2e, q, qf);
+  if (tA < thd) {
+    while (true) {
+      load_raw_tile(kh, vh, min(tB, tcl), S, a, q, R1);
+      const int tC = take_tile(&next_tile, lane);
+      consume_raw_tile<false>(R0, st, tA, S, A.scale_log2e, q, qf);
+      if (tB >= thd) break;
+      load_raw_tile(kh, vh, min(tC, tcl), S, a, q, R0);
+      const int tD = take_tile(&next_tile, lane);
+      consume_raw_tile<false>(R1, st, tB, S, A.scale_log2e, q, qf);
+      if (tC >= thd) break;
+      tA = tC; tB = tD;
     }
   }
-  if (own_partial) {
+  if (part_here && wave == 0) {
     load_raw_tile(kh, vh, ntiles - 1, S, a, q, R0);
     consume_raw_tile<true>(R0, st, ntiles - 1, S, A.scale_log2e, q, qf);
   }
@@ -812,6 +836,10 @@ __global__ void __launch_bounds__(256, 2) k_bf16_attn_split(const AttnArgs A) {
 
 using namespace gaac;
 
+#ifdef GAAC_PHASE_TIMING
+static long long* g_dbg = nullptr;
+extern "C" void gaac_set_phase_buffer(long long* p) { g_dbg = p; }
+#endif
 static int attn_split_impl(
     const uint8_t* smk, const uint8_t* ck, const int* fk, const int* tok, const uint8_t* ovk, const int* ohsk, const uint8_t* b3k, const uint8_t* b4k,
     const uint8_t* smv, const uint8_t* cv, const int* fv, const int* tov, const uint8_t* ovv, const int* ohsv, const uint8_t* b3v, const uint8_t* b4v,
@@ -835,9 +863,12 @@ static int attn_split_impl(
   A.tickets = tickets; A.out = (u16*)out;
   GAAC_REQUIRE(!tickets || out, "gaac_attn: the fused merge needs an output buffer");
   A.pool = nullptr; A.raw = nullptr; A.mt = nullptr; A.bt = nullptr; A.bt_stride = 0; A.TS = 0;
+#ifdef GAAC_PHASE_TIMING
+  A.dbg = g_dbg;
+#endif
   // few blocks: one 8-wave block per CU (half as many partials); otherwise two 4-wave blocks per CU
-  if ((long)B * n_kv * nslot <= 256) hipLaunchKernelGGL((k_attn_split<false, 8>), dim3(B * n_kv, nslot), dim3(512), 0, (hipStream_t)stream, A);
-  else hipLaunchKernelGGL((k_attn_split<false, 4>), dim3(B * n_kv, nslot), dim3(256), 0, (hipStream_t)stream, A);
+  if ((long)B * n_kv * nslot <= 256) hipLaunchKernelGGL((k_attn_split<false, 8>), dim3(B * n_kv * nslot), dim3(512), 0, (hipStream_t)stream, A);
+  else hipLaunchKernelGGL((k_attn_split<false, 4>), dim3(B * n_kv * nslot), dim3(256), 0, (hipStream_t)stream, A);
   return launch_status("gaac_attn(split)");
 }
 
@@ -901,8 +932,11 @@ extern "C" int gaac_paged_attn(
   A.kt = nullptr; A.vt = nullptr; A.tl = nullptr; A.tcap = 0;
   A.tickets = tickets; A.out = (u16*)out;
   A.pool = pool; A.raw = (const u16*)raw; A.mt = mt; A.bt = bt; A.bt_stride = bt_stride; A.TS = TS;
-  if ((long)B * n_kv * nsplit <= 256) hipLaunchKernelGGL((k_attn_split<true, 8>), dim3(B * n_kv, nsplit), dim3(512), 0, (hipStream_t)stream, A);
-  else hipLaunchKernelGGL((k_attn_split<true, 4>), dim3(B * n_kv, nsplit), dim3(256), 0, (hipStream_t)stream, A);
+#ifdef GAAC_PHASE_TIMING
+  A.dbg = nullptr;
+#endif
+  if ((long)B * n_kv * nsplit <= 256) hipLaunchKernelGGL((k_attn_split<true, 8>), dim3(B * n_kv * nsplit), dim3(512), 0, (hipStream_t)stream, A);
+  else hipLaunchKernelGGL((k_attn_split<true, 4>), dim3(B * n_kv * nsplit), dim3(256), 0, (hipStream_t)stream, A);
   return launch_status("gaac_paged_attn");
 }
 
