@@ -336,7 +336,9 @@ struct WaveState { f32x4 acc[8]; float m_run, mu_run, l_run; };     // acc[i][r]
 
 // unit decode with the escape contribution already expanded to exponent-field words x (see AttnLds::xlut)
 __device__ __forceinline__ void decode_unit_x(u32 slo, u32 shi, u32 g24, const u32x4& x, const u32x4& bw, u32* __restrict__ out) {
-  const u32 cw = (g24 & 0xFFFu) | ((g24 << 4) & 0x0FFF0000u);
+  // low-half codes stay at bits 3p, high-half codes move to bits 16 + 3p; the bits this leaves at 12..15 and 28..31 never reach the
+  // fields the four masks below keep
+  const u32 cw = ((g24 << 4) & 0x0FFF0000u) | (g24 & ~0x0FFF0000u);
   const u32 c0 = (cw << 7) & 0x03800380u, c1 = (cw << 4) & 0x03800380u, c2 = (cw << 1) & 0x03800380u, c3 = (cw >> 2) & 0x03800380u;
   // bw: the base words of the unit's tier (3-bit base, or 4-bit base for promoted and raw groups: their x holds hi5 - base4)
   const u32 e0 = c0 + bw[0] + x[0], e1 = c1 + bw[1] + x[1], e2 = c2 + bw[2] + x[2], e3 = c3 + bw[3] + x[3];
@@ -483,10 +485,10 @@ __device__ __forceinline__ int take_tile(int* ctr, int lane) {
 template <bool PAGED, int NW>
 __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const AttnArgs A) {
   constexpr int NT = 64 * NW;
-  __shared__ AttnLds L;
-  __shared__ MergeLds<NW> M;
-  __shared__ int2 tile_table[PAGED ? MAX_CHUNK : 1];
-  __shared__ int next_tile;
+  // one LDS object so that the tables the tile loop reads sit at the lowest addresses (immediate offsets of the LDS loads)
+  struct BlockLds { AttnLds L; int next_tile; int2 tile_table[PAGED ? MAX_CHUNK : 1]; MergeLds<NW> M; };
+  __shared__ BlockLds lds;
+  AttnLds& L = lds.L; MergeLds<NW>& M = lds.M; int2* tile_table = lds.tile_table; int& next_tile = lds.next_tile;
   const int tid = threadIdx.x;
   GAAC_STAMP(0);
   // One-dimensional grid.  With a raw tail there is one more block per (row, kv head): those are dispatched first, own no compressed

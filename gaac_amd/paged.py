@@ -60,7 +60,9 @@ class LayerState:
 
     @staticmethod
     def pool_bytes(num_blocks: int, n_kv: int, ovf_slot: int = 128) -> int:
-        return num_blocks * 2 * n_kv * (OVF_OFF + ovf_slot)
+        """Bytes of the block pool: the slots plus 16 bytes of slack (the attention kernel fetches a lane's escape bytes as one
+        unaligned 8-byte load, which may reach up to 7 bytes past the last slot)."""
+        return num_blocks * 2 * n_kv * (OVF_OFF + ovf_slot) + 16
 
     @property
     def bases(self):

@@ -99,7 +99,8 @@ int gaac_cache_append(
 /* ---- paged slot pool (the layout of /root/reference/gaac/vllm/paged_kernel.py:3-6 and store.py:17-19) -------------------------------
  * pool: tile slots of TS bytes, physical tile p = block*2*n_kv + 2*kvh + kind: [0,2048) sign/mantissa | [2048,2816) codes |
  * [2816,2880) 16 tag words | [2880,TS) escape bytes.  mt int32 [num_blocks*2*n_kv]: p = compressed in its slot, ~r = raw BF16 tile r of
- * raw [tiles][16][128].  stack/top: free raw tiles; err: failed pops.  Bases uint8 [n_kv,128]. */
+ * raw [tiles][16][128].  stack/top: free raw tiles; err: failed pops.  Bases uint8 [n_kv,128].  The pool allocation must extend at
+ * least 8 bytes past its last slot (escape bytes are fetched with unaligned 8-byte loads). */
 
 /* LayerState.store -> _store_tiles, store.py:22-105.  key/value: bf16 rows [num_tokens][n_kv][128] with row strides in elements;
  * ent int32 [n_ent][4] = (block, first token row, offset in block, rows), block < 0 = inactive; freeq int32 [n_ent*2*n_kv] receives
