@@ -103,6 +103,7 @@ def test_prefill_then_decode_steps_through_a_permuted_block_table():
     assert int(P.st.top) == 64 - n_raw and n_raw >= filling * 2 * N_KV
     P.check([0, 1, 2, 3], randn_bf16((4, N_KV * G, 128), seed=77, scale=0.1), nsplit=1)
     P.check([0, 1, 2, 3], randn_bf16((4, N_KV * G, 128), seed=78, scale=0.1), nsplit=7)
+    P.check([0, 1, 2, 3], randn_bf16((4, N_KV * G, 128), seed=79, scale=0.1), nsplit=20)      # 320 blocks: the four-wave block shape
 
 
 def test_tiles_whose_escapes_do_not_fit_stay_raw_and_blocks_are_released():
