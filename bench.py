@@ -3,7 +3,7 @@
   python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A step = one layer's decode attention (ONE kernel: split pass incl. the 7-token BF16 tail, merged by the last block of each
-kv head) for config 1 of BASELINE.json:
+kv head) for the headline configuration:
 32 query heads over 8 kv heads (GQA group 4), head_dim 128, 65536 compressed tokens + 7 tail tokens, batch 1.
 Inputs are synthetic (seeded, CPU generator), encoded once with the HIP encoder and resident in HBM before timing.
 Successive steps rotate over distinct copies of the compressed KV so the 256 MB Infinity Cache cannot serve them.

@@ -2,15 +2,19 @@
 // Counterpart of gaac_attn / gaac_tail / gaac_combine / gaac_attn_launch in /root/reference/gaac/kernel.py:48-326
 // (same inputs, same partial (m, l, acc) protocol, same slot map and padded-row behaviour), redesigned for CDNA4:
 //
-//   * one block = (batch row, kv head, split), 4 waves; wave w streams tiles tlo+w, tlo+w+4, ... of the split;
+//   * one block = (batch row, kv head, split), 8 waves (one block per CU) for launches of up to 256 blocks, else 4 waves (two per CU);
+//     the waves of a block take their tiles from a counter in LDS (the two waves sharing a SIMD would otherwise finish far apart);
 //   * scores   S[16 tok x 16 heads]  = K[16 x 128] . Q^T      : 4 x v_mfma_f32_16x16x32_bf16   (A = decoded K units)
 //   * output   O^T[128 x 16 heads]  += V^T[128 x 16] . P^T     : 8 x v_mfma_f32_16x16x16_bf16   (A = decoded V units)
 //     The score tile lands in the register layout the second product wants for P^T, so P never crosses lanes.
 //   * the GQA group (<= 16 query heads) rides in the N dimension; register use does not depend on it;
-//   * three-stage prefetch per wave: tag words of tile t+8, payload + escape bytes of tile t+4, consume tile t;
-//   * rows that are not compressed (the raw BF16 tail of a cache head, <= 16 tokens) are one extra block row of the same launch
-//     (dispatched first): a block without tiles whose fifth block-merge partial holds the tail; it writes partial slot nsplit.  Softmax runs in base 2 (scale * log2 e
-//     folded into the scores).
+//   * three-stage prefetch per wave: tag words two tiles ahead, payload + escape bytes one tile ahead, consume;
+//   * rows that are not compressed (the raw BF16 tail of a cache head, <= 16 tokens) are extra blocks of the same launch
+//     (dispatched first): blocks without tiles whose extra block-merge partial holds the tail; they write partial slot nsplit;
+//   * the last block of a (row, kv head) to publish its partial merges all of them (fused gaac_combine); k_attn_combine is the
+//     two-launch alternative;
+//   * k_attn_split<true, .> reads the paged slot pool through block and mode tables (paged_kernel.py:42-241).
+//   Softmax runs in base 2 (scale * log2 e folded into the scores).
 #include "gaac_tile.h"
 #include "gaac_capi.h"
 #include "../../include/gaac_hip.h"
