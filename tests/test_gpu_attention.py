@@ -88,6 +88,25 @@ def test_uncompressed_baseline_kernel(B, n_kv, G, S):
             assert np.abs(got[b] - ref[b]).max() <= 2e-2 * np.abs(ref[b]).max() + 1e-3, (b, ns)
 
 
+def test_random_shapes_lengths_and_split_counts():
+    """Seeded sweep over ragged lengths (partly filled last tile, fewer tiles than waves or splits), group sizes and split counts,
+    through both block shapes (launches above 256 blocks use four-wave blocks)."""
+    dev = require_gpu()
+    from gaac_amd import attention
+    rng = np.random.default_rng(123)
+    for case in range(24):
+        B, n_kv = int(rng.integers(1, 4)), int(rng.choice([1, 2, 3, 8]))
+        G = int(rng.choice([1, 2, 3, 5, 7, 8, 12, 16]))
+        S = int(rng.choice([1, 15, 16, 17, 31, 100, 129, 500, 700]))
+        ns = int(rng.choice([1, 2, 3, 9, 40, 130]))
+        k16, v16, kp, vp = _pages(B, n_kv, S, dev, seed=1000 + case)
+        q16 = randn_bf16((B, n_kv * G, 128), seed=2000 + case, scale=0.2)
+        got = O.bf16_to_f32(to_u16(attention(to_bf16(q16, dev), kp, vp, SCALE, nsplit=ns)))
+        ref = _ref(q16, k16, v16, B, n_kv)
+        for b in range(B):
+            assert np.abs(got[b] - ref[b]).max() <= 2e-2 * np.abs(ref[b]).max() + 1e-3, (case, B, n_kv, G, S, ns, b)
+
+
 def test_stated_tolerance_on_unit_scale_data():
     """max-abs <= 1e-2 and mean-abs <= 1e-3 against decompress + fp32 softmax attention, q ~ N(0,1)."""
     dev = require_gpu()

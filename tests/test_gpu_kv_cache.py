@@ -131,3 +131,39 @@ def test_overflow_is_flagged_not_written():
     with pytest.raises(RuntimeError, match="escape stream"):
         cache.check_capacity()
     assert int(cache.k.ovf_used.max()) == 0 and int(cache.k.flags.abs().max()) == 0
+
+
+@pytest.mark.parametrize("n_kv,G", [(1, 16), (8, 1), (2, 6)])
+def test_other_head_shapes_with_random_batches(n_kv, G):
+    """Per-sequence bases, random prompt lengths (incl. shorter than one tile), random batches with padded rows, 50 decode steps."""
+    dev = require_gpu()
+    from gaac_amd import CompressedKVCache
+    rng = np.random.default_rng(n_kv * 100 + G)
+    n_slots = 5
+    cache = CompressedKVCache(n_slots=n_slots, n_kv=n_kv, capacity=300)
+    tok = lambda x16: np.ascontiguousarray(x16.transpose(1, 0, 2))
+    hist = {}
+    for s in range(n_slots):
+        L = int(rng.choice([1, 7, 16, 33, 150]))
+        k16, v16 = tok(kv_like16(n_kv, L, seed=10 + s, scale_seed=77)), tok(kv_like16(n_kv, L, seed=60 + s, scale_seed=78))
+        cache.prefill(s, to_bf16(k16, dev), to_bf16(v16, dev)); hist[s] = (k16, v16)
+    for step in range(50):
+        slots_l = [int(x) for x in rng.permutation(n_slots)[:3]] + [-1]
+        rng.shuffle(slots_l)
+        k16, v16 = tok(kv_like16(n_kv, 4, seed=500 + step, scale_seed=77)), tok(kv_like16(n_kv, 4, seed=900 + step, scale_seed=78))
+        cache.append(torch.tensor(slots_l, dtype=torch.int32, device=dev), to_bf16(k16, dev), to_bf16(v16, dev))
+        for b, s in enumerate(slots_l):
+            if s >= 0: hist[s] = (np.concatenate([hist[s][0], k16[b:b + 1]]), np.concatenate([hist[s][1], v16[b:b + 1]]))
+        if step % 16 == 15: cache.check_capacity()
+        if step % 17 == 0 or step == 49:
+            q16 = randn_bf16((4, n_kv * G, 128), seed=300 + step, scale=0.1)
+            out = O.bf16_to_f32(to_u16(cache.attention(to_bf16(q16, dev), torch.tensor(slots_l, dtype=torch.int32, device=dev), SCALE)))
+            for b, s in enumerate(slots_l):
+                if s < 0:
+                    assert np.abs(out[b]).max() == 0
+                    continue
+                ref = O.ref_attention(q16[b], hist[s][0], hist[s][1], SCALE)
+                assert np.abs(out[b] - ref).max() <= 2e-2 * np.abs(ref).max() + 1e-3, (step, b, s)
+    for s in range(n_slots):
+        dk, dv = cache.decompress(s)
+        assert np.array_equal(to_u16(dk), hist[s][0]) and np.array_equal(to_u16(dv), hist[s][1])
