@@ -122,9 +122,15 @@ __global__ void __launch_bounds__(64) k_decode_tiles(const uint8_t* __restrict__
   const int brow = bidx ? bidx[h] : h % n_kv;
   const long row0 = (long)h * S_pad + (long)tile * T;
   // rows beyond S carry tag 0 (the encoder writes every word of a tile) and are not written
-  decode_tile_rows<KIND>(sm + row0 * D, cd + row0 * CB, flags + row0, ovf + head_start[h] + tile_off[(long)h * (S_pad / T) + tile],
-                         base3 + (long)brow * D, base4 + (long)brow * D, lane, min(T, S - tile * T),
-                         out + (long)h * out_head_stride + (long)tile * T * out_row_stride, out_row_stride);
+  __shared__ __align__(16) u16 stage[T * D];
+  u16* dst = out + (long)h * out_head_stride + (long)tile * T * out_row_stride;
+  const uint8_t* esc = ovf + head_start[h] + tile_off[(long)h * (S_pad / T) + tile];
+  if ((out_row_stride & 7) == 0 && (reinterpret_cast<uintptr_t>(dst) & 15) == 0)
+    decode_tile_staged<KIND>(sm + row0 * D, cd + row0 * CB, flags + row0, esc, base3 + (long)brow * D, base4 + (long)brow * D, lane,
+                             min(T, S - tile * T), stage, dst, out_row_stride);
+  else      // rows that are not 16-byte aligned: element stores
+    decode_tile_rows<KIND>(sm + row0 * D, cd + row0 * CB, flags + row0, esc, base3 + (long)brow * D, base4 + (long)brow * D, lane,
+                           min(T, S - tile * T), dst, out_row_stride);
 }
 
 // Plain streaming copy with the access shape of the attention kernel's payload loads (16 B per lane, 1 KiB per wave-wide

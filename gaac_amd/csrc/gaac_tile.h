@@ -148,4 +148,20 @@ __device__ __forceinline__ void decode_tile_rows(const uint8_t* __restrict__ sm_
   }
 }
 
+// decode_tile_rows through an LDS staging tile (T*D u16, owned by the calling wave): the channel permutation turns the decoder's
+// output into 2-byte scattered stores, which LDS absorbs; global memory then gets 16-byte stores, a full 256-byte row per 16 lanes.
+template <int KIND>
+__device__ __forceinline__ void decode_tile_staged(const uint8_t* __restrict__ sm_tile, const uint8_t* __restrict__ cd_tile,
+                                                   const int* __restrict__ flags_tile, const uint8_t* __restrict__ esc,
+                                                   const uint8_t* __restrict__ b3row, const uint8_t* __restrict__ b4row, int lane, int nvalid,
+                                                   u16* __restrict__ stage, u16* __restrict__ out, long row_stride) {
+  decode_tile_rows<KIND>(sm_tile, cd_tile, flags_tile, esc, b3row, b4row, lane, T, stage, D);
+  wave_lds_sync();
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int idx = k * 64 + lane, row = idx >> 4, c16 = idx & 15;
+    if (row < nvalid) *reinterpret_cast<u32x4*>(out + (long)row * row_stride + c16 * 8) = *reinterpret_cast<const u32x4*>(stage + row * D + c16 * 8);
+  }
+}
+
 }  // namespace gaac

@@ -130,10 +130,19 @@ __global__ void __launch_bounds__(64) k_paged_decode(const PagedDecodeArgs A) {
     return;
   }
   const uint8_t* slot = A.pool + (long)m * A.TS;
-  if (kind) decode_tile_rows<KIND_V>(slot, slot + SLOT_CD, reinterpret_cast<const int*>(slot + SLOT_FL), slot + SLOT_OV,
-                                     A.b3v + (long)kvh * D, A.b4v + (long)kvh * D, lane, nvalid, out, A.row_stride);
-  else decode_tile_rows<KIND_K>(slot, slot + SLOT_CD, reinterpret_cast<const int*>(slot + SLOT_FL), slot + SLOT_OV,
-                                A.b3k + (long)kvh * D, A.b4k + (long)kvh * D, lane, nvalid, out, A.row_stride);
+  __shared__ __align__(16) u16 stage[T * D];
+  const bool aligned = (A.row_stride & 7) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
+  if (kind) {
+    if (aligned) decode_tile_staged<KIND_V>(slot, slot + SLOT_CD, reinterpret_cast<const int*>(slot + SLOT_FL), slot + SLOT_OV,
+                                            A.b3v + (long)kvh * D, A.b4v + (long)kvh * D, lane, nvalid, stage, out, A.row_stride);
+    else decode_tile_rows<KIND_V>(slot, slot + SLOT_CD, reinterpret_cast<const int*>(slot + SLOT_FL), slot + SLOT_OV,
+                                  A.b3v + (long)kvh * D, A.b4v + (long)kvh * D, lane, nvalid, out, A.row_stride);
+  } else {
+    if (aligned) decode_tile_staged<KIND_K>(slot, slot + SLOT_CD, reinterpret_cast<const int*>(slot + SLOT_FL), slot + SLOT_OV,
+                                            A.b3k + (long)kvh * D, A.b4k + (long)kvh * D, lane, nvalid, stage, out, A.row_stride);
+    else decode_tile_rows<KIND_K>(slot, slot + SLOT_CD, reinterpret_cast<const int*>(slot + SLOT_FL), slot + SLOT_OV,
+                                  A.b3k + (long)kvh * D, A.b4k + (long)kvh * D, lane, nvalid, out, A.row_stride);
+  }
 }
 
 }  // namespace gaac
