@@ -142,6 +142,10 @@ def test_other_head_shapes_with_random_batches(n_kv, G):
     n_slots = 5
     cache = CompressedKVCache(n_slots=n_slots, n_kv=n_kv, capacity=300)
     tok = lambda x16: np.ascontiguousarray(x16.transpose(1, 0, 2))
+    def kv_like16(H, L, seed, scale_seed=None):      # unit-scale values (spread-out softmax weights) with sparse far-off ones
+        x = randn_bf16((H, L, 128), seed=seed)
+        x[:, ::5, 3::29] = 0x3580
+        return x
     hist = {}
     for s in range(n_slots):
         L = int(rng.choice([1, 7, 16, 33, 150]))
@@ -156,7 +160,7 @@ def test_other_head_shapes_with_random_batches(n_kv, G):
             if s >= 0: hist[s] = (np.concatenate([hist[s][0], k16[b:b + 1]]), np.concatenate([hist[s][1], v16[b:b + 1]]))
         if step % 16 == 15: cache.check_capacity()
         if step % 17 == 0 or step == 49:
-            q16 = randn_bf16((4, n_kv * G, 128), seed=300 + step, scale=0.1)
+            q16 = randn_bf16((4, n_kv * G, 128), seed=300 + step, scale=1.0)
             out = O.bf16_to_f32(to_u16(cache.attention(to_bf16(q16, dev), torch.tensor(slots_l, dtype=torch.int32, device=dev), SCALE)))
             for b, s in enumerate(slots_l):
                 if s < 0:
