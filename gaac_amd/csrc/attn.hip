@@ -9,8 +9,8 @@
 //     The score tile lands in the register layout the second product wants for P^T, so P never crosses lanes.
 //   * the GQA group (<= 16 query heads) rides in the N dimension; register use does not depend on it;
 //   * three-stage prefetch per wave: tag words two tiles ahead, payload + escape bytes one tile ahead, consume;
-//   * rows that are not compressed (the raw BF16 tail of a cache head, <= 16 tokens) are extra blocks of the same launch
-//     (dispatched first): blocks without tiles whose extra block-merge partial holds the tail; they write partial slot nsplit;
+//   * the raw BF16 tail of a cache head (<= 16 tokens) is attended by one wave of the block that owns the last split, as an extra
+//     partial of that block's merge; the wave then joins the tile hand-out, so the other waves absorb the tiles it did not take;
 //   * the last block of a (row, kv head) to publish its partial merges all of them (fused gaac_combine); k_attn_combine is the
 //     two-launch alternative;
 //   * k_attn_split<true, .> reads the paged slot pool through block and mode tables (paged_kernel.py:42-241).
@@ -206,6 +206,60 @@ __device__ __forceinline__ void raw_rows_attend(RawScratch& R, const u16* __rest
     float acc = acc5[g][d] * R.alpha[g];
     for (int tk = 0; tk < nvalid; ++tk) acc += R.sc[g][tk] * bf16_bits_to_float(vrows[tk * D + d]);
     acc5[g][d] = acc;
+  }
+}
+
+// The same for ONE wave and rows in global memory: the raw tail of a cache head is attended by wave 0 of the block that owns the last
+// split, before that wave joins the block's tile hand-out (the other waves pick up the tiles it does not get to).  No block barrier.
+// Lane (t = lane >> 2, c = lane & 3) takes row t, channels 32c .. 32c+31 for the scores; lane owns output dims 2*lane, 2*lane+1.
+__device__ __forceinline__ void wave_rows_attend(float (*__restrict__ sc)[T], const u16* __restrict__ krows, const u16* __restrict__ vrows,
+                                                 int nvalid, const u16* __restrict__ qrows, float scale_log2e, int G, int lane,
+                                                 float* __restrict__ m5, float* __restrict__ l5, float (*__restrict__ acc5)[D]) {
+  const int t = lane >> 2, c = lane & 3;
+  float kr[32];
+  {
+    u32x4 kv[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) kv[j] = t < nvalid ? *reinterpret_cast<const u32x4*>(krows + t * D + 32 * c + 8 * j) : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) { kr[8 * j + 2 * i] = bf16_bits_to_float(kv[j][i] & 0xFFFFu); kr[8 * j + 2 * i + 1] = bf16_bits_to_float(kv[j][i] >> 16); }
+  }
+  for (int g = 0; g < G; ++g) {
+    float d = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const u32x4 qv = *reinterpret_cast<const u32x4*>(qrows + g * D + 32 * c + 8 * j);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) d += bf16_bits_to_float(qv[i] & 0xFFFFu) * kr[8 * j + 2 * i] + bf16_bits_to_float(qv[i] >> 16) * kr[8 * j + 2 * i + 1];
+    }
+    d += __shfl_xor(d, 1, 64); d += __shfl_xor(d, 2, 64);
+    if (c == 0) sc[g][t] = t < nvalid ? d * scale_log2e : -INFINITY;
+  }
+  wave_lds_sync();
+  for (int g = lane >> 4; g < G; g += 4) {      // 16 lanes per head: softmax over the row
+    const int tk = lane & 15;
+    const float s = sc[g][tk];
+    float mt = s;
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) mt = fmaxf(mt, __shfl_xor(mt, o, 16));
+    const float p = __builtin_amdgcn_exp2f(s - (mt == -INFINITY ? 0.f : mt));
+    float lt = p;
+#pragma unroll
+    for (int o = 8; o > 0; o >>= 1) lt += __shfl_xor(lt, o, 16);
+    sc[g][tk] = p;
+    if (tk == 0) { m5[g] = mt; l5[g] = lt; }
+  }
+  wave_lds_sync();
+  u32 vv[T];
+#pragma unroll
+  for (int tk = 0; tk < T; ++tk) vv[tk] = tk < nvalid ? *reinterpret_cast<const u32*>(vrows + tk * D + 2 * lane) : 0u;
+  for (int g = 0; g < G; ++g) {
+    float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+    for (int tk = 0; tk < T; ++tk) { const float p = sc[g][tk]; a0 += p * bf16_bits_to_float(vv[tk] & 0xFFFFu); a1 += p * bf16_bits_to_float(vv[tk] >> 16); }
+    acc5[g][2 * lane] = a0; acc5[g][2 * lane + 1] = a1;
   }
 }
 
@@ -495,12 +549,9 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
   AttnLds& L = lds.L; MergeLds<NW>& M = lds.M; int2* tile_table = lds.tile_table; int& next_tile = lds.next_tile;
   const int tid = threadIdx.x;
   GAAC_STAMP(0);
-  // One-dimensional grid.  With a raw tail there is one more block per (row, kv head): those are dispatched first, own no compressed
-  // tile and write partial slot nsplit.  The other blocks are numbered split-fastest, so the splits of one kv head go round the
-  // eight XCDs (workgroups are dealt to XCDs in turn) instead of all landing on one: heads with heavier tiles then load every XCD alike.
-  const int n_bh = (int)gridDim.x / A.nslot, n_tail = A.nslot > A.nsplit ? n_bh : 0;
-  const int lin = (int)blockIdx.x - n_tail;
-  const int bh = lin < 0 ? (int)blockIdx.x : lin / A.nsplit, split = lin < 0 ? A.nsplit : lin % A.nsplit;
+  // One-dimensional grid, numbered split-fastest: the splits of one kv head go round the eight XCDs (workgroups are dealt to XCDs in
+  // turn) instead of all landing on one, so heads with heavier tiles load every XCD alike.
+  const int bh = (int)blockIdx.x / A.nsplit, split = (int)blockIdx.x % A.nsplit;
   const int b = bh / A.n_kv, kvh = bh % A.n_kv, G = A.G;
   const int slot = PAGED ? 0 : A.slot[b], ch = PAGED ? kvh : (slot < 0 ? 0 : slot) * A.n_kv + kvh;
   const long qh0 = (long)b * A.n_q + (long)kvh * G;
@@ -564,6 +615,17 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
   for (int i = 0; i < 8; ++i) st.acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
   st.m_run = -INFINITY; st.mu_run = 0.f; st.l_run = 0.f;
 
+  // ---- the raw tail of the cache head: wave 0 of the last split's block, before it joins the tile hand-out
+  if (!PAGED && A.kt && split == A.nsplit - 1 && wave == 0) {
+    const int TL = slot < 0 ? 0 : min(A.tl[ch], A.tcap);
+    if (TL > 0) {
+      // probabilities go through this wave's own merge slot: the other waves write theirs as soon as they run out of tiles
+      float (*sc)[T] = reinterpret_cast<float (*)[T]>(&M.acc[0][0][0]);
+      wave_rows_attend(sc, A.kt + (long)ch * A.tcap * D, A.vt + (long)ch * A.tcap * D, TL, A.q + qh0 * D, A.scale_log2e, G, lane,
+                       M.m[NW], M.l[NW], M.acc[NW]);
+    }
+  }
+
   if (tA < thd) {
     int tC = take_tile(&next_tile, lane);
     while (true) {        // R0 = tile tA, Tg = tags of tile tB
@@ -592,8 +654,8 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
     load_tile<PAGED>(B, t, lane, Tg, R0);
     if (!PAGED || !Tg.raw) consume<PAGED, true>(R0, st, L, B, Tg.kto, Tg.vto, t, S, A.scale_log2e, a, q, qf);
   }
-  // ---- rows kept as plain BF16: the raw tail of a cache head (the extra block row) or, in the paged pool, tiles of this split
-  // whose K or V side is a raw tile (the block that is still filling, or escapes that did not fit the slot)
+  // ---- paged pool: tiles of this split whose K or V side is a raw tile (the block that is still filling, or escapes that did not
+  // fit the slot) are attended by the whole block
   if (PAGED) {
     bool mine = false;
     for (int i = tid; i < thi - tlo; i += NT) mine |= (tile_table[i].x | tile_table[i].y) < 0;
@@ -621,13 +683,6 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
         __syncthreads();      // staging rows are free again
       }
     }
-  } else if (split == A.nsplit) {
-    RawScratch& R = *reinterpret_cast<RawScratch*>(&M.acc[0][0][0]);
-    const int TL = slot < 0 ? 0 : min(A.tl[ch], A.tcap);
-    for (int g = tid >> 7; g < G; g += NT / 128) M.acc[NW][g][tid & 127] = 0.f;
-    raw_rows_begin<NT>(R, A, qh0, G, tid);
-    raw_rows_attend<NT>(R, A.kt + (long)ch * A.tcap * D, A.vt + (long)ch * A.tcap * D, TL, A.scale_log2e, G, tid, M.m[NW], M.l[NW], M.acc[NW]);
-    __syncthreads();      // the scratch view is dead before the waves publish into the same memory
   }
   // The accumulators are MFMA results: keep their first non-MFMA read a full MFMA latency away on every path.
   asm volatile("s_nop 7\n\ts_nop 7" ::: "memory");
@@ -857,8 +912,8 @@ static int attn_split_impl(
   GAAC_REQUIRE(B > 0 && S_pad > 0 && S_pad % T == 0 && NB > 0, "gaac_attn: bad sizes B=%d S_pad=%d NB=%d", B, S_pad, NB);
   const bool has_tail = kt != nullptr;
   GAAC_REQUIRE(!has_tail || (vt && TL && TCAP >= 1 && TCAP <= T), "gaac_attn: tail needs kt, vt, TL and 1 <= TCAP <= %d", T);
-  const int nslot = nsplit + (has_tail ? 1 : 0);
-  GAAC_REQUIRE(nsplit >= 1 && nslot <= MAX_SLOTS, "gaac_attn: nsplit must be in 1..%d", MAX_SLOTS - 1);
+  const int nslot = nsplit;
+  GAAC_REQUIRE(nsplit >= 1 && nslot <= MAX_SLOTS, "gaac_attn: nsplit must be in 1..%d", MAX_SLOTS);
   AttnArgs A;
   A.k = StoreView{smk, ck, fk, tok, ovk, ohsk, b3k, b4k};
   A.v = StoreView{smv, cv, fv, tov, ovv, ohsv, b3v, b4v};
@@ -903,7 +958,7 @@ extern "C" int gaac_attn_launch(
   int rc = attn_split_impl(smk, ck, fk, tok, ovk, ohsk, b3k, b4k, smv, cv, fv, tov, ovv, ohsv, b3v, b4v, q, slot, B, n_q, n_kv, SL, S_pad,
                            scale, nsplit, NB, kt, vt, TL, TCAP, pm, pl, pa, nullptr, nullptr, stream);
   if (rc) return rc;
-  return gaac_attn_combine(pm, pl, pa, out, B * n_q, nsplit + (kt ? 1 : 0), stream);
+  return gaac_attn_combine(pm, pl, pa, out, B * n_q, nsplit, stream);
 }
 
 extern "C" int gaac_attn_fused(

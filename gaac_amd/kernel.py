@@ -10,7 +10,7 @@ from . import _lib
 
 D = 128
 GMAX = 16
-MAX_SPLITS = 1023
+MAX_SPLITS = 1024
 
 
 def _ext():
@@ -23,12 +23,6 @@ def choose_nsplit(B: int, n_kv: int, S: int, target_ctas: int = 256, min_tok: in
     part, kernel.py:340-342), at least min_tok tokens per split.  Launches of up to 256 blocks use eight-wave blocks, larger
     ones four-wave blocks (two per CU)."""
     return min(max(1, target_ctas // (B * n_kv)), max(1, S // min_tok), cap)
-
-
-def nsplit_with_tail_row(nsplit: int, B: int, n_kv: int, resident: int = 256) -> int:
-    """The raw tail adds one block row to the launch: give up one split when that row would no longer be resident together with the
-    others (one eight-wave block on each of the 256 CUs), so that no block has to wait for a free CU."""
-    return nsplit - 1 if nsplit > 1 and B * n_kv * nsplit <= resident < B * n_kv * (nsplit + 1) else nsplit
 
 
 class AttnWorkspace:
@@ -60,7 +54,7 @@ def attn_launch(K, V, q2d, slots, n_q, n_kv, SL, S_pad, scale, nsplit, kt=None, 
         raise RuntimeError("head_dim must be 128")
     B = slots.shape[0]
     has_tail = kt is not None and kt.numel() > 0
-    nslot = nsplit + (1 if has_tail else 0)
+    nslot = nsplit        # the raw tail is folded into the last split's partial
     if ws is None:
         ws = AttnWorkspace(B * n_q, nslot, q2d.dtype, q2d.device)
     elif ws.rows != B * n_q or ws.nslot != nslot:

@@ -12,7 +12,7 @@ import torch
 from . import _lib
 from .codec import Codec, Page, D, T, CB, TILE_MAX_ESC, row_offsets
 from .encoder import TileEncoder
-from .kernel import _ext, choose_nsplit, nsplit_with_tail_row, attn_launch, AttnWorkspace
+from .kernel import _ext, choose_nsplit, attn_launch, AttnWorkspace
 
 TAIL = 16
 ROW_BYTES = D + CB + 4          # sign/mantissa + codes + tag word of one token row
@@ -134,10 +134,10 @@ class CompressedKVCache:
     def attention(self, q: torch.Tensor, slots: torch.Tensor, scale: float, max_len: int | None = None, nsplit: int | None = None):
         """q: [B, n_q, D] bf16 (row b attends over slot slots[b]) -> [B, n_q, D] bf16."""
         B, n_q, _ = q.shape
-        if nsplit is None: nsplit = nsplit_with_tail_row(choose_nsplit(B, self.n_kv, max_len or self.cap), B, self.n_kv)
+        if nsplit is None: nsplit = choose_nsplit(B, self.n_kv, max_len or self.cap)
         ws = self._partials.get((B, n_q, nsplit))
         if ws is None:
-            ws = self._partials[(B, n_q, nsplit)] = AttnWorkspace(B * n_q, nsplit + 1, q.dtype, q.device, with_out=False)
+            ws = self._partials[(B, n_q, nsplit)] = AttnWorkspace(B * n_q, nsplit, q.dtype, q.device, with_out=False)
         out = attn_launch(self.k, self.v, q.reshape(B * n_q, D).contiguous(), slots, n_q, self.n_kv, self.S, self.cap, scale, nsplit,
                           self.k.tail, self.v.tail, self.tail_len, TAIL, ws=ws)
         return out.view(B, n_q, D)

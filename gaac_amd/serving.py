@@ -168,7 +168,6 @@ class DecodeRunner:
         self.slots = torch.arange(B, dtype=torch.int32, device=dev)
         self.dlens = self.lens[:B].clone()
         self.nsplit = nsplit or choose_nsplit(B, self.cfg.n_kv_heads, self.cfg.max_len)
-        if self.kv == "gaac" and nsplit is None: self.nsplit = max(1, self.nsplit - 1)       # the tail block row takes one row of resident blocks
         self.logits = None
         self.graph = None
         if not use_graph: return

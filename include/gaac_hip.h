@@ -54,7 +54,7 @@ int gaac_decode_tiles(int kind, const uint8_t* sm, const uint8_t* codes, const i
  * head, nsplit, and the optional raw tail kt/vt [cache heads, TCAP, 128] bf16 with lengths TL (kt == NULL: no tail).
  * NB = rows of the base tables (n_kv, or the number of cache heads for per-sequence bases).
  * Differences from the reference entry: the caller passes the partial buffers pm, pl [B*n_q*NSLOT] and
- * pa [B*n_q*NSLOT*128] (fp32, NSLOT = nsplit + (kt != NULL)) and `out` [B*n_q, 128] bf16 instead of having them
+ * pa [B*n_q*NSLOT*128] (fp32, NSLOT = nsplit; the tail is folded into the last split's partial) and `out` [B*n_q, 128] bf16 instead of having them
  * allocated inside; GQA group sizes 1..16 are accepted (reference: 1..8). */
 int gaac_attn_launch(
     const uint8_t* smk, const uint8_t* ck, const int* fk, const int* tok, const uint8_t* ovk, const int* ohsk, const uint8_t* b3k, const uint8_t* b4k,
