@@ -425,8 +425,33 @@ def bench_phases(a):
     m = np.median(np.array(rows), 0)
     names = ["last_block_start", "first_tile_loads_issued_mean", "tables_ready_mean", "loop_end_waves_0_3_mean", f"loop_end_waves_{NW - 4}_{NW - 1}_mean",
              "block_loop_end_mean", "block_loop_end_max", "partial_stored_mean", "partial_stored_max", "last_stamp", "loop_end_fastest_xcd_mean", "loop_end_slowest_xcd_mean"]
+    # the same launches back to back (one HIP graph, a stamp buffer per launch): what the idle gap between dependent launches is and
+    # how the phases move when arguments and metadata are still cached from the launch before
+    nb2b = 24
+    dbgs = torch.zeros(nb2b, nblk * 16, dtype=torch.int64, device=dev)
+    def chain():
+        for i in range(nb2b):
+            lib.gaac_set_phase_buffer(dbgs[i].data_ptr()); f(i)
+    st = torch.cuda.Stream(); st.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(st): chain()
+    torch.cuda.current_stream().wait_stream(st); torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g): chain()
+    b2b = []
+    for _ in range(5):
+        dbgs.zero_(); torch.cuda.synchronize(); g.replay(); torch.cuda.synchronize()
+        raw = dbgs.cpu().numpy().astype(np.float64) * 0.01
+        t = raw[:, :nblk * 8].reshape(nb2b, nblk, 8); wv = raw[:, nblk * 8:].reshape(nb2b, nblk, 8)[:, :, :NW]
+        first, last = t[:, :, 0].min(1), t[:, :, 5].max(1)
+        for i in range(4, nb2b - 1):
+            b2b.append([first[i + 1] - first[i], first[i + 1] - last[i], last[i] - first[i], (t[i, :, 1] - first[i]).mean(),
+                        (wv[i].max(1) - first[i]).mean(), (wv[i].max(1) - first[i]).max(), (t[i, :, 4] - first[i]).max()])
+    mb = np.median(np.array(b2b), 0)
+    lib.gaac_set_phase_buffer(None)
+    bnames = ["period", "idle_gap_between_launches", "first_entry_to_last_stamp", "tables_ready_mean", "block_loop_end_mean", "block_loop_end_max", "partial_stored_max"]
     print(json.dumps({"workload": "config 1 kernel phases, us from the first block's entry (median of 20 launches, each after a device synchronize)",
-                      "nsplit": nsplit, "waves_per_block": NW, **{k: round(float(v), 2) for k, v in zip(names, m)}}))
+                      "nsplit": nsplit, "waves_per_block": NW, **{k: round(float(v), 2) for k, v in zip(names, m)},
+                      "back_to_back_in_one_graph": {k: round(float(v), 2) for k, v in zip(bnames, mb)}}))
 
 
 if __name__ == "__main__":

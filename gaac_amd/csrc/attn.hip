@@ -280,26 +280,28 @@ struct AttnLds {
 template <int NW> struct MergeLds { float m[NW + 1][GMAX], l[NW + 1][GMAX]; float acc[NW + 1][GMAX][D]; };
 static_assert(sizeof(RawScratch) <= 4 * GMAX * D * sizeof(float) && MAX_SLOTS <= GMAX * D, "scratch views must fit the merge buffer");
 struct TableRegs { u32 b0, b1; u32 qlo[4], qhi[4]; };      // one thread's raw inputs of the per-block tables
-// global loads only (issued before the first tile's loads so that the two latencies overlap)
-__device__ __forceinline__ void tables_load(TableRegs& Tr, int tid, const AttnArgs& A, int brow, long qh0) {
-  {   // one base word per thread: kind = tid >> 7, tier = (tid >> 6) & 1, group = (tid >> 2) & 15, p = tid & 3
-    const int kind = tid >> 7, tier = (tid >> 6) & 1, g = (tid >> 2) & 15, p = tid & 3;
-    const StoreView& st = kind ? A.v : A.k;
-    const uint8_t* row = (tier ? st.base4 : st.base3) + (long)brow * D;
-    const int c0 = kind ? chan_v(8 * g + p) : chan_k(8 * g + p), c1 = kind ? chan_v(8 * g + p + 4) : chan_k(8 * g + p + 4);
-    Tr.b0 = row[c0]; Tr.b1 = row[c1];
-  }
+// Global loads only, in two parts so that each can be issued as soon as its address is known (the query rows need the batch row, the
+// base rows the cache head) and waited for only when the tables are written.
+__device__ __forceinline__ void tables_load_q(TableRegs& Tr, int tid, const u16* __restrict__ qrows, int G) {
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {      // query words: head = idx >> 6, group = (idx >> 2) & 15, p = idx & 3
-    const int idx = tid + 256 * k, h = idx >> 6, g = (idx >> 2) & 15, p = idx & 3;
-    Tr.qlo[k] = 0u; Tr.qhi[k] = 0u;
-    if (h < A.G) {
-      const u16* qp = A.q + (qh0 + h) * D;
-      Tr.qlo[k] = qp[chan_k(8 * g + p)]; Tr.qhi[k] = qp[chan_k(8 * g + p + 4)];
-    }
+  for (int k = 0; k < 4; ++k) {      // query words: head = idx >> 6, group = (idx >> 2) & 15, p = idx & 3 (heads >= G: any valid row)
+    const int idx = tid + 256 * k, h = min(idx >> 6, G - 1), g = (idx >> 2) & 15, p = idx & 3;
+    const u16* qp = qrows + h * D;
+    Tr.qlo[k] = qp[chan_k(8 * g + p)]; Tr.qhi[k] = qp[chan_k(8 * g + p + 4)];
   }
 }
-__device__ __forceinline__ void tables_store(AttnLds& L, const TableRegs& Tr, int tid) {
+__device__ __forceinline__ void tables_load_bases(TableRegs& Tr, int tid, const uint8_t* k3, const uint8_t* k4, const uint8_t* v3,
+                                                  const uint8_t* v4, int brow) {
+  // one base word per thread: kind = tid >> 7, tier = (tid >> 6) & 1, group = (tid >> 2) & 15, p = tid & 3
+  const int kind = tid >> 7, tier = (tid >> 6) & 1, g = (tid >> 2) & 15, p = tid & 3;
+  const uint8_t* row = (kind ? (tier ? v4 : v3) : (tier ? k4 : k3)) + (long)brow * D;
+  const int c0 = kind ? chan_v(8 * g + p) : chan_k(8 * g + p), c1 = kind ? chan_v(8 * g + p + 4) : chan_k(8 * g + p + 4);
+  Tr.b0 = row[c0]; Tr.b1 = row[c1];
+}
+__device__ __forceinline__ void tables_store(AttnLds& L, TableRegs Tr, int tid, int G) {
+  // the loaded values are first needed HERE: keeps the compiler from packing them (and waiting for them) where they were loaded
+  asm volatile("" : "+v"(Tr.b0), "+v"(Tr.b1), "+v"(Tr.qlo[0]), "+v"(Tr.qlo[1]), "+v"(Tr.qlo[2]), "+v"(Tr.qlo[3]), "+v"(Tr.qhi[0]),
+               "+v"(Tr.qhi[1]), "+v"(Tr.qhi[2]), "+v"(Tr.qhi[3]));
   {
     const u32 e = (u32)tid;
     u32x4 w;
@@ -323,7 +325,7 @@ __device__ __forceinline__ void tables_store(AttnLds& L, const TableRegs& Tr, in
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
     const int idx = tid + 256 * k, h = idx >> 6, g = (idx >> 2) & 15, p = idx & 3;
-    reinterpret_cast<u32*>(&L.qw[h][g])[p] = Tr.qlo[k] | (Tr.qhi[k] << 16);
+    reinterpret_cast<u32*>(&L.qw[h][g])[p] = h < G ? Tr.qlo[k] | (Tr.qhi[k] << 16) : 0u;
   }
 }
 
@@ -531,12 +533,15 @@ __device__ __forceinline__ void consume(const TileRegs& R, WaveState& st, const 
     consume_tile<PAGED, PARTIAL, false>(R, st, L, B, kto, vto, tile, S, scale_log2e, a, q, qf);
 }
 
-// next tile index from the block's counter (one LDS atomic per wave, the result is uniform)
-__device__ __forceinline__ int take_tile(int* ctr, int lane) {
+// Next tile for a wave from the block's counter in LDS (lane 0's value counts).  The caller makes it uniform only when it needs it,
+// one tile later, so that no wave waits for the LDS atomic.  Indices past the block's range come back as NO_TILE.
+constexpr int NO_TILE = 0x3FFFFFFF;
+__device__ __forceinline__ int take_tile(int* ctr, int hi, int lane) {
   int v = 0;
-  if (lane == 0) v = atomicAdd(ctr, 1);
-  return __builtin_amdgcn_readfirstlane(v);
+  if (lane == 0) { v = atomicAdd(ctr, 1); v = v < hi ? v : NO_TILE; }
+  return v;
 }
+__device__ __forceinline__ int uniform_tile(int v) { return __builtin_amdgcn_readfirstlane(v); }
 
 // ---------------------------------------------------------------------------------------------------- main kernel
 // NW = waves per block: 4 (two blocks per CU) or 8 (one block per CU: half as many partials to merge for the same occupancy)
@@ -551,14 +556,35 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
   GAAC_STAMP(0);
   // One-dimensional grid, numbered split-fastest: the splits of one kv head go round the eight XCDs (workgroups are dealt to XCDs in
   // turn) instead of all landing on one, so heads with heavier tiles load every XCD alike.
+  // The start of a block is a chain of dependent loads (arguments -> slot -> lengths and stream starts -> tag words -> escape bytes),
+  // each a trip to memory with nothing else to do: issue everything a level allows before the first use of any of its results.
+  // Level 0: the kernel arguments, forced into scalar registers together (otherwise each is fetched where it is first used).
+  if (PAGED)
+    asm volatile("" ::"s"(A.q), "s"(A.sl), "s"(A.bt), "s"(A.mt), "s"(A.pool), "s"(A.raw), "s"(A.k.base3), "s"(A.k.base4), "s"(A.v.base3),
+                 "s"(A.v.base4), "s"(A.nsplit), "s"(A.n_kv), "s"(A.n_q), "s"(A.G), "s"(A.NB), "s"(A.bt_stride), "s"(A.TS));
+  else
+    asm volatile("" ::"s"(A.q), "s"(A.slot), "s"(A.sl), "s"(A.k.sm), "s"(A.k.cd), "s"(A.k.flags), "s"(A.k.tile_off), "s"(A.k.ovf),
+                 "s"(A.k.head_start), "s"(A.k.base3), "s"(A.k.base4), "s"(A.v.sm), "s"(A.v.cd), "s"(A.v.flags), "s"(A.v.tile_off),
+                 "s"(A.v.ovf), "s"(A.v.head_start), "s"(A.v.base3), "s"(A.v.base4), "s"(A.kt), "s"(A.tl), "s"(A.nsplit), "s"(A.n_kv),
+                 "s"(A.n_q), "s"(A.G), "s"(A.NB), "s"(A.S_pad), "s"(A.tcap));
   const int bh = (int)blockIdx.x / A.nsplit, split = (int)blockIdx.x % A.nsplit;
   const int b = bh / A.n_kv, kvh = bh % A.n_kv, G = A.G;
-  const int slot = PAGED ? 0 : A.slot[b], ch = PAGED ? kvh : (slot < 0 ? 0 : slot) * A.n_kv + kvh;
   const long qh0 = (long)b * A.n_q + (long)kvh * G;
+  // Level 1: the slot of the batch row; the query rows do not depend on it
   TableRegs Tr;
-  if (tid < 256) tables_load(Tr, tid, A, ch % A.NB, qh0);
+  if (tid < 256) tables_load_q(Tr, tid, A.q + qh0 * D, G);
+  const int slot = PAGED ? 0 : A.slot[b], ch = PAGED ? kvh : (slot < 0 ? 0 : slot) * A.n_kv + kvh;
+  // Level 2: everything indexed by the cache head
+  int S, TLh = 0; long khs = 0, vhs = 0;
+  if (PAGED) S = max(A.sl[b], 0);
+  else {
+    S = A.sl[ch]; khs = A.k.head_start[ch]; vhs = A.v.head_start[ch];
+    TLh = (A.kt ? A.tl : A.sl)[ch];            // no branch between the loads of this level
+    if (slot < 0) S = 0;
+    if (slot < 0 || !A.kt) TLh = 0;
+  }
+  if (tid < 256) tables_load_bases(Tr, tid, A.k.base3, A.k.base4, A.v.base3, A.v.base4, ch % A.NB);
 
-  const int S = PAGED ? max(A.sl[b], 0) : (slot < 0 ? 0 : A.sl[ch]);
   const int ntiles = (S + T - 1) / T, chunk = PAGED ? min((ntiles + A.nsplit - 1) / A.nsplit, MAX_CHUNK) : (ntiles + A.nsplit - 1) / A.nsplit;
   const int tlo = min(split * chunk, ntiles), thi = min(tlo + chunk, ntiles);
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, a = lane & 15, q = lane >> 4;
@@ -575,8 +601,8 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
     __syncthreads();
   } else {
     const long rowb = (long)ch * A.S_pad, tileb = (long)ch * (A.S_pad / T);
-    B.ksm = A.k.sm + rowb * D; B.kcd = A.k.cd + rowb * CB; B.kfl = A.k.flags + rowb; B.kto = A.k.tile_off + tileb; B.kov = A.k.ovf + A.k.head_start[ch];
-    B.vsm = A.v.sm + rowb * D; B.vcd = A.v.cd + rowb * CB; B.vfl = A.v.flags + rowb; B.vto = A.v.tile_off + tileb; B.vov = A.v.ovf + A.v.head_start[ch];
+    B.ksm = A.k.sm + rowb * D; B.kcd = A.k.cd + rowb * CB; B.kfl = A.k.flags + rowb; B.kto = A.k.tile_off + tileb; B.kov = A.k.ovf + khs;
+    B.vsm = A.v.sm + rowb * D; B.vcd = A.v.cd + rowb * CB; B.vfl = A.v.flags + rowb; B.vto = A.v.tile_off + tileb; B.vov = A.v.ovf + vhs;
     B.TS = 0;
   }
 
@@ -599,7 +625,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
   }
   if (tid == 0) next_tile = tlo + 2 * NW;
   GAAC_STAMP(6);
-  if (tid < 256) tables_store(L, Tr, tid);
+  if (tid < 256) tables_store(L, Tr, tid, G);
   GAAC_STAMP(7);
   if (tid < GMAX) { M.m[NW][tid] = -INFINITY; M.l[NW][tid] = 0.f; }
   __syncthreads();        // block tables are ready
@@ -617,7 +643,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
 
   // ---- the raw tail of the cache head: wave 0 of the last split's block, before it joins the tile hand-out
   if (!PAGED && A.kt && split == A.nsplit - 1 && wave == 0) {
-    const int TL = slot < 0 ? 0 : min(A.tl[ch], A.tcap);
+    const int TL = min(TLh, A.tcap);
     if (TL > 0) {
       // probabilities go through this wave's own merge slot: the other waves write theirs as soon as they run out of tiles
       float (*sc)[T] = reinterpret_cast<float (*)[T]>(&M.acc[0][0][0]);
@@ -627,21 +653,23 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
   }
 
   if (tA < thd) {
-    int tC = take_tile(&next_tile, lane);
+    int vC = take_tile(&next_tile, thd, lane);
     while (true) {        // R0 = tile tA, Tg = tags of tile tB
       TgC1 = Tg;
       load_tile<PAGED>(B, min(tB, tcl), lane, Tg, R1);
-      const int tD = take_tile(&next_tile, lane);
+      const int vD = take_tile(&next_tile, thd, lane);
+      const int tC = uniform_tile(vC);
       load_tags<PAGED>(B, TT, min(tC, tcl), a, Tg);
       if (!PAGED || !TgC0.raw) consume<PAGED, false>(R0, st, L, B, TgC0.kto, TgC0.vto, tA, S, A.scale_log2e, a, q, qf);
       if (tB >= thd) break;
       TgC0 = Tg;
       load_tile<PAGED>(B, min(tC, tcl), lane, Tg, R0);
-      const int tE = take_tile(&next_tile, lane);
+      const int vE = take_tile(&next_tile, thd, lane);
+      const int tD = uniform_tile(vD);
       load_tags<PAGED>(B, TT, min(tD, tcl), a, Tg);
       if (!PAGED || !TgC1.raw) consume<PAGED, false>(R1, st, L, B, TgC1.kto, TgC1.vto, tB, S, A.scale_log2e, a, q, qf);
       if (tC >= thd) break;
-      tA = tC; tB = tD; tC = tE;
+      tA = tC; tB = tD; vC = vE;
     }
   }
   GAAC_STAMP(2);
@@ -850,11 +878,11 @@ __global__ void __launch_bounds__(256, 2) k_bf16_attn_split(const AttnArgs A) {
   if (tA < thd) {
     while (true) {
       load_raw_tile(kh, vh, min(tB, tcl), S, a, q, R1);
-      const int tC = take_tile(&next_tile, lane);
+      const int tC = uniform_tile(take_tile(&next_tile, thd, lane));
       consume_raw_tile<false>(R0, st, tA, S, A.scale_log2e, q, qf);
       if (tB >= thd) break;
       load_raw_tile(kh, vh, min(tC, tcl), S, a, q, R0);
-      const int tD = take_tile(&next_tile, lane);
+      const int tD = uniform_tile(take_tile(&next_tile, thd, lane));
       consume_raw_tile<false>(R1, st, tB, S, A.scale_log2e, q, qf);
       if (tC >= thd) break;
       tA = tC; tB = tD;
