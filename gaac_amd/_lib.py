@@ -15,7 +15,7 @@ _SIGNATURES = {
     "gaac_bases_from_hist": [P, c_int, P, P, P],
     "gaac_encode_tiles": [c_int, P, c_int, c_int, c_int, c_int, P, P, c_int, P, P, P, P, P, P, P],
     "gaac_compact": [P, P, P, P, P, c_int, c_int, P],
-    "gaac_row_offsets": [P, c_int, c_int, c_int, P, P],
+    "gaac_row_offsets": [P, c_int, c_int, c_int, P, P, P],
     "gaac_decode_tiles": [c_int, P, P, P, P, P, P, P, P, c_int, P, c_int, c_int, c_int, P, c_long, c_long, P],
     "gaac_attn_split": [P] * 16 + [P, P, c_int, c_int, c_int, P, c_int, c_float, c_int, c_int, P, P, P, c_int, P, P, P, P],
     "gaac_attn_combine": [P, P, P, P, c_int, c_int, P],

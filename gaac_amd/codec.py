@@ -106,7 +106,8 @@ def row_offsets(flags: torch.Tensor, S: int) -> torch.Tensor:
     H, S_pad = flags.shape
     out = torch.empty(H, S, dtype=torch.int32, device=flags.device)
     if S:
-        _lib.call("gaac_row_offsets", _lib.ptr(flags), H, S, S_pad, _lib.ptr(out), _lib.stream())
+        sums = torch.empty(H * ((S + 2047) // 2048), dtype=torch.int32, device=flags.device)
+        _lib.call("gaac_row_offsets", _lib.ptr(flags), H, S, S_pad, _lib.ptr(sums), _lib.ptr(out), _lib.stream())
     return out
 
 
@@ -128,7 +129,7 @@ def encode_page(x: torch.Tensor, kind: str, base3: torch.Tensor, base4: torch.Te
     head_bytes = tile_bytes.sum(1)
     head_start = torch.cat([torch.zeros(1, dtype=torch.int64, device=dev), torch.cumsum(head_bytes, 0)]).to(torch.int32).contiguous()
     ovf = torch.zeros(int(head_start[-1]) + 8, dtype=torch.uint8, device=dev)
-    tile_off = (torch.cumsum(tile_bytes, 1) - tile_bytes).to(torch.int32).contiguous()
+    tile_off = torch.empty_like(tile_bytes)
     _lib.call("gaac_compact", _lib.ptr(slots), _lib.ptr(tile_bytes), _lib.ptr(tile_off), _lib.ptr(head_start), _lib.ptr(ovf),
               H, ntiles, _lib.stream())
     return Page(sm, cd, flags, row_offsets(flags, S), ovf, head_start, tile_off, base3, base4, H, S, n_kv, kind)

@@ -33,21 +33,23 @@ __device__ __forceinline__ void append_one(const CacheStore& st, const u16* __re
   for (int k = 0; k < 4; ++k) {
     const int idx = k * 64 + lane, row = idx >> 4, c16 = idx & 15;
     const u16* src = row < T - 1 ? tail_h + row * D : xrow;
-    *reinterpret_cast<u32x4*>(&L.x[row * D + c16 * 8]) = *reinterpret_cast<const u32x4*>(src + c16 * 8);
+    *reinterpret_cast<u32x4*>(&L.x[row * XROW + c16 * 8]) = *reinterpret_cast<const u32x4*>(src + c16 * 8);
   }
   const int brow = h % A.NB;
   stage_bases(L, st.base3 + (long)brow * D, st.base4 + (long)brow * D, lane);
   wave_lds_sync();
+  BaseRegs Bs;
+  load_base_regs<KIND>(L, lane & 15, lane >> 4, Bs);
   const long row0 = (long)h * A.cap + (long)tile * T;
   uint8_t* sm_tile = st.sm + row0 * D; uint8_t* cd_tile = st.cd + row0 * CB; int* fl_tile = st.flags + row0;
   const int used = st.ovf_used[h];
   uint8_t* dst = st.ovf + (long)h * A.ovf_cap + used;
   int total; bool fits = true;
-  if (used + TILE_MAX_ESC + 8 <= A.ovf_cap) total = encode_staged_tile<KIND>(L, T, lane, sm_tile, cd_tile, fl_tile, dst);
+  if (used + TILE_MAX_ESC + 8 <= A.ovf_cap) total = encode_staged_tile<KIND>(L, Bs, T, lane, sm_tile, cd_tile, fl_tile, dst);
   else {      // less than one worst-case tile of room: count first, write only what fits
-    total = encode_staged_tile<KIND>(L, T, lane, sm_tile, cd_tile, fl_tile, nullptr);
+    total = encode_staged_tile<KIND>(L, Bs, T, lane, sm_tile, cd_tile, fl_tile, nullptr);
     fits = used + total + 8 <= A.ovf_cap;
-    if (fits) encode_staged_tile<KIND>(L, T, lane, sm_tile, cd_tile, fl_tile, dst);
+    if (fits) encode_staged_tile<KIND>(L, Bs, T, lane, sm_tile, cd_tile, fl_tile, dst);
   }
   if (fits) {
     if (lane == 0) { st.tile_off[(long)h * (A.cap / T) + tile] = used; st.ovf_used[h] = used + total; }

@@ -50,44 +50,104 @@ __global__ void __launch_bounds__(128) k_bases_from_hist(const long long* __rest
 }
 
 // ---------------------------------------------------------------------------------------------------- page encoder
+// A block of four waves takes 16 consecutive tiles of one head, wave w the tiles w, w+4, w+8, w+12 of them (one-wave blocks, one per
+// tile, would be limited by the rate at which workgroups can be launched).  The rows of a wave's next tile are fetched into
+// registers while it encodes the current one.
+constexpr int CODEC_WAVES = 4, CODEC_TPW = 4, CODEC_TPB = CODEC_WAVES * CODEC_TPW;
 template <int KIND>
-__global__ void __launch_bounds__(64) k_encode_tiles(const u16* __restrict__ x, int S, int S_in, int S_pad, const uint8_t* __restrict__ base3,
-                                                     const uint8_t* __restrict__ base4, int n_kv, const int* __restrict__ bidx,
-                                                     uint8_t* __restrict__ sm, uint8_t* __restrict__ cd, int* __restrict__ flags,
-                                                     uint8_t* __restrict__ esc_slots, int* __restrict__ tile_bytes, int ntiles) {
-  __shared__ EncodeLds L;
-  const int tile = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+__global__ void __launch_bounds__(64 * CODEC_WAVES) k_encode_tiles(const u16* __restrict__ x, int S, int S_in, int S_pad,
+                                                                   const uint8_t* __restrict__ base3, const uint8_t* __restrict__ base4,
+                                                                   int n_kv, const int* __restrict__ bidx, uint8_t* __restrict__ sm,
+                                                                   uint8_t* __restrict__ cd, int* __restrict__ flags,
+                                                                   uint8_t* __restrict__ esc_slots, int* __restrict__ tile_bytes, int ntiles) {
+  __shared__ EncodeLds Ls[CODEC_WAVES];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, h = blockIdx.y;
+  EncodeLds& L = Ls[wave];
   const int brow = bidx ? bidx[h] : h % n_kv;
-  const int nvalid = min(T, S - tile * T);
-  stage_rows(L, x + ((long)h * S_in + (long)tile * T) * D, D, nvalid, lane);
+  int tile = blockIdx.x * CODEC_TPB + wave;
+  if (tile >= ntiles) return;
+  const u16* xh = x + (long)h * S_in * D;
+  RowRegs R, Rn;
+  load_rows(R, xh + (long)tile * T * D, D, min(T, S - tile * T), lane);
   stage_bases(L, base3 + (long)brow * D, base4 + (long)brow * D, lane);
+  wave_lds_sync();
+  BaseRegs Bs;                // the base words of the lane's units: the same for every tile of the head
+  load_base_regs<KIND>(L, lane & 15, lane >> 4, Bs);
+  for (int i = 0; i < CODEC_TPW && tile < ntiles; ++i, tile += CODEC_WAVES) {
+    const int nvalid = min(T, S - tile * T), next = tile + CODEC_WAVES;
+    store_rows(L, R, lane);
+    if (i + 1 < CODEC_TPW && next < ntiles) load_rows(Rn, xh + (long)next * T * D, D, min(T, S - next * T), lane);
+    wave_lds_sync();
+    const long row0 = (long)h * S_pad + (long)tile * T;
+    const int total = encode_staged_tile<KIND>(L, Bs, nvalid, lane, sm + row0 * D, cd + row0 * CB, flags + row0,
+                                               esc_slots + ((long)h * ntiles + tile) * TILE_MAX_ESC);
+    if (lane == 0) tile_bytes[(long)h * ntiles + tile] = total;
+    wave_lds_sync();          // the staged rows and tag words are free again
+    R = Rn;
+  }
+}
+
+// Packs the per-tile escape slots into the head's stream and writes the tile offsets (exclusive sum of the tile sizes of the head).
+// A block takes 64 consecutive tiles: it sums the sizes of all earlier tiles of the head itself (a few thousand integers at most),
+// scans its own 64 and copies, one wave per tile: most tiles hold a few dozen escape bytes.
+constexpr int COMPACT_TPB = 64;
+__global__ void __launch_bounds__(256) k_compact(const uint8_t* __restrict__ esc_slots, const int* __restrict__ tile_bytes,
+                                                 int* __restrict__ tile_off, const int* __restrict__ head_start,
+                                                 uint8_t* __restrict__ ovf, int ntiles) {
+  __shared__ int part[4];
+  __shared__ int offs[COMPACT_TPB];
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, h = blockIdx.y, t0 = blockIdx.x * COMPACT_TPB;
+  const int* tb = tile_bytes + (long)h * ntiles;
+  int before = 0;
+  for (int i = tid; i < t0; i += 256) before += tb[i];
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) before += __shfl_xor(before, o, 64);
+  if (lane == 0) part[wave] = before;
   __syncthreads();
-  const long row0 = (long)h * S_pad + (long)tile * T;
-  const int total = encode_staged_tile<KIND>(L, nvalid, lane, sm + row0 * D, cd + row0 * CB, flags + row0,
-                                             esc_slots + ((long)h * ntiles + tile) * TILE_MAX_ESC);
-  if (lane == 0) tile_bytes[(long)h * ntiles + tile] = total;
+  if (wave == 0) {
+    const int n = t0 + lane < ntiles ? tb[t0 + lane] : 0;
+    int incl = n;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) { const int v = __shfl_up(incl, o, 64); if (lane >= o) incl += v; }
+    const int off = part[0] + part[1] + part[2] + part[3] + incl - n;
+    offs[lane] = off;
+    if (t0 + lane < ntiles) tile_off[(long)h * ntiles + t0 + lane] = off;
+  }
+  __syncthreads();
+  const int hs = head_start[h];
+  for (int k = wave; k < COMPACT_TPB && t0 + k < ntiles; k += 4) {
+    const long i = (long)h * ntiles + t0 + k;
+    const int n = tb[t0 + k];
+    const uint8_t* src = esc_slots + i * TILE_MAX_ESC;
+    uint8_t* dst = ovf + hs + offs[k];
+    for (int j = lane; j < n; j += 64) dst[j] = src[j];
+  }
 }
 
-__global__ void __launch_bounds__(64) k_compact(const uint8_t* __restrict__ esc_slots, const int* __restrict__ tile_bytes,
-                                                const int* __restrict__ tile_off, const int* __restrict__ head_start,
-                                                uint8_t* __restrict__ ovf, int ntiles) {
-  const int tile = blockIdx.x, h = blockIdx.y;
-  const long i = (long)h * ntiles + tile;
-  const int n = tile_bytes[i];
-  const uint8_t* src = esc_slots + i * TILE_MAX_ESC;
-  uint8_t* dst = ovf + head_start[h] + tile_off[i];
-  for (int k = threadIdx.x; k < n; k += 64) dst[k] = src[k];
-}
-
-// One block per (head, chunk of 2048 tag words): the bytes of all earlier chunks are re-summed by the block itself (a few hundred KB
-// out of L2 at most), then the chunk is scanned: 8 words per thread serially, thread totals by a block scan.
+// Two passes over the tag words of a head: escape bytes per chunk of 2048 rows, then per chunk the bytes of all earlier chunks (a
+// short sum) plus a scan inside the chunk: 8 words per thread serially, thread totals by a block scan.
 constexpr int RO_CHUNK = 2048;
-__global__ void __launch_bounds__(256) k_row_offsets(const int* __restrict__ flags, int S, int S_pad, int* __restrict__ out) {
+__global__ void __launch_bounds__(256) k_row_chunk_sums(const int* __restrict__ flags, int S, int S_pad, int* __restrict__ chunk_sums) {
+  __shared__ int sh[4];
+  const int h = blockIdx.y, c = blockIdx.x, tid = threadIdx.x;
+  const int* f = flags + (long)h * S_pad;
+  const int s0 = c * RO_CHUNK + tid * 8;
+  int mine = 0;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) mine += s0 + k < S ? esc_bytes((u32)f[s0 + k]) : 0;
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) mine += __shfl_xor(mine, o, 64);
+  if ((tid & 63) == 0) sh[tid >> 6] = mine;
+  __syncthreads();
+  if (tid == 0) chunk_sums[(long)h * gridDim.x + c] = sh[0] + sh[1] + sh[2] + sh[3];
+}
+__global__ void __launch_bounds__(256) k_row_offsets(const int* __restrict__ flags, int S, int S_pad, const int* __restrict__ chunk_sums,
+                                                     int* __restrict__ out) {
   __shared__ int sh[256];
   const int h = blockIdx.y, c = blockIdx.x, tid = threadIdx.x;
   const int* f = flags + (long)h * S_pad;
   int before = 0;
-  for (int s = tid; s < c * RO_CHUNK; s += 256) before += esc_bytes((u32)f[s]);
+  for (int i = tid; i < c; i += 256) before += chunk_sums[(long)h * gridDim.x + i];
   const int s0 = c * RO_CHUNK + tid * 8;
   int rb[8], mine = 0;
 #pragma unroll
@@ -112,6 +172,8 @@ __global__ void __launch_bounds__(256) k_row_offsets(const int* __restrict__ fla
 }
 
 // ---------------------------------------------------------------------------------------------------- page decoder
+// One wave per tile: short-lived waves at full occupancy overlap the dependent loads of a tile (tag words -> escape bytes) with the
+// arithmetic and the stores of others (four tiles in a row per wave were a third slower).
 template <int KIND>
 __global__ void __launch_bounds__(64) k_decode_tiles(const uint8_t* __restrict__ sm, const uint8_t* __restrict__ cd, const int* __restrict__ flags,
                                                      const int* __restrict__ tile_off, const uint8_t* __restrict__ ovf,
@@ -122,7 +184,7 @@ __global__ void __launch_bounds__(64) k_decode_tiles(const uint8_t* __restrict__
   const int brow = bidx ? bidx[h] : h % n_kv;
   const long row0 = (long)h * S_pad + (long)tile * T;
   // rows beyond S carry tag 0 (the encoder writes every word of a tile) and are not written
-  __shared__ __align__(16) u16 stage[T * D];
+  __shared__ __align__(16) u16 stage[T * STAGE_ROW];
   u16* dst = out + (long)h * out_head_stride + (long)tile * T * out_row_stride;
   const uint8_t* esc = ovf + head_start[h] + tile_off[(long)h * (S_pad / T) + tile];
   if ((out_row_stride & 7) == 0 && (reinterpret_cast<uintptr_t>(dst) & 15) == 0)
@@ -171,22 +233,24 @@ int gaac_encode_tiles(int kind, const void* x, int H, int S, int S_in, int S_pad
   GAAC_REQUIRE(H > 0 && S > 0 && S_in >= S && S_pad >= (S + T - 1) / T * T && S_pad % T == 0 && n_kv > 0,
                "gaac_encode_tiles: bad sizes H=%d S=%d S_in=%d S_pad=%d n_kv=%d", H, S, S_in, S_pad, n_kv);
   const int ntiles = (S + T - 1) / T;
-  dim3 grid(ntiles, H);
-  if (kind == 0) hipLaunchKernelGGL(k_encode_tiles<KIND_K>, grid, dim3(64), 0, (hipStream_t)stream, (const u16*)x, S, S_in, S_pad, base3, base4, n_kv, bidx, sm, codes, flags, esc_slots, tile_bytes, ntiles);
-  else hipLaunchKernelGGL(k_encode_tiles<KIND_V>, grid, dim3(64), 0, (hipStream_t)stream, (const u16*)x, S, S_in, S_pad, base3, base4, n_kv, bidx, sm, codes, flags, esc_slots, tile_bytes, ntiles);
+  dim3 grid((ntiles + CODEC_TPB - 1) / CODEC_TPB, H);
+  if (kind == 0) hipLaunchKernelGGL(k_encode_tiles<KIND_K>, grid, dim3(64 * CODEC_WAVES), 0, (hipStream_t)stream, (const u16*)x, S, S_in, S_pad, base3, base4, n_kv, bidx, sm, codes, flags, esc_slots, tile_bytes, ntiles);
+  else hipLaunchKernelGGL(k_encode_tiles<KIND_V>, grid, dim3(64 * CODEC_WAVES), 0, (hipStream_t)stream, (const u16*)x, S, S_in, S_pad, base3, base4, n_kv, bidx, sm, codes, flags, esc_slots, tile_bytes, ntiles);
   return launch_status("gaac_encode_tiles");
 }
 
-int gaac_compact(const uint8_t* esc_slots, const int* tile_bytes, const int* tile_off, const int* head_start, uint8_t* ovf,
+int gaac_compact(const uint8_t* esc_slots, const int* tile_bytes, int* tile_off, const int* head_start, uint8_t* ovf,
                  int H, int ntiles, void* stream) {
   GAAC_REQUIRE(esc_slots && tile_bytes && tile_off && head_start && ovf && H > 0 && ntiles > 0, "gaac_compact: bad arguments");
-  hipLaunchKernelGGL(k_compact, dim3(ntiles, H), dim3(64), 0, (hipStream_t)stream, esc_slots, tile_bytes, tile_off, head_start, ovf, ntiles);
+  hipLaunchKernelGGL(k_compact, dim3((ntiles + COMPACT_TPB - 1) / COMPACT_TPB, H), dim3(256), 0, (hipStream_t)stream, esc_slots, tile_bytes, tile_off, head_start, ovf, ntiles);
   return launch_status("gaac_compact");
 }
 
-int gaac_row_offsets(const int* flags, int H, int S, int S_pad, int* out, void* stream) {
-  GAAC_REQUIRE(flags && out && H > 0 && S > 0 && S_pad >= S, "gaac_row_offsets: bad arguments");
-  hipLaunchKernelGGL(k_row_offsets, dim3((S + RO_CHUNK - 1) / RO_CHUNK, H), dim3(256), 0, (hipStream_t)stream, flags, S, S_pad, out);
+int gaac_row_offsets(const int* flags, int H, int S, int S_pad, int* chunk_sums, int* out, void* stream) {
+  GAAC_REQUIRE(flags && out && chunk_sums && H > 0 && S > 0 && S_pad >= S, "gaac_row_offsets: bad arguments");
+  const dim3 grid((S + RO_CHUNK - 1) / RO_CHUNK, H);
+  hipLaunchKernelGGL(k_row_chunk_sums, grid, dim3(256), 0, (hipStream_t)stream, flags, S, S_pad, chunk_sums);
+  hipLaunchKernelGGL(k_row_offsets, grid, dim3(256), 0, (hipStream_t)stream, flags, S, S_pad, chunk_sums, out);
   return launch_status("gaac_row_offsets");
 }
 

@@ -8,22 +8,36 @@
 namespace gaac {
 
 // LDS scratch of one encoding wave
+constexpr int XROW = D + 8;     // staged row stride in elements: 16 padding bytes spread the sixteen rows of a column over the banks
 struct EncodeLds {
-  u16 x[T * D];        // the tile's BF16 bit patterns, token-major, natural channel order (rows >= nvalid are zero)
+  u16 x[T * XROW];     // the tile's BF16 bit patterns, token-major, natural channel order (rows >= nvalid are zero)
   uint8_t b3[D], b4[D];
   u32 tags[T];
   int rowoff[T + 1];   // exclusive prefix of per-row escape bytes; [16] = tile total
 };
 
-// Stage 16 rows of 128 BF16 (row r at src + r*row_stride elements) into lds.x; rows >= nvalid read as zero.
-__device__ __forceinline__ void stage_rows(EncodeLds& L, const u16* __restrict__ src, long row_stride, int nvalid, int lane) {
+// 16 rows of 128 BF16 (row r at src + r*row_stride elements): lane's four 16-byte pieces; rows >= nvalid read as zero.
+struct RowRegs { u32x4 v[4]; };
+__device__ __forceinline__ void load_rows(RowRegs& R, const u16* __restrict__ src, long row_stride, int nvalid, int lane) {
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
-    int idx = k * 64 + lane, row = idx >> 4, c16 = idx & 15;
-    u32x4 v = {0u, 0u, 0u, 0u};
-    if (row < nvalid) v = *reinterpret_cast<const u32x4*>(src + (long)row * row_stride + c16 * 8);
-    *reinterpret_cast<u32x4*>(&L.x[row * D + c16 * 8]) = v;
+    const int idx = k * 64 + lane, row = idx >> 4, c16 = idx & 15;
+    R.v[k] = u32x4{0u, 0u, 0u, 0u};
+    if (row < nvalid) R.v[k] = *reinterpret_cast<const u32x4*>(src + (long)row * row_stride + c16 * 8);
   }
+}
+__device__ __forceinline__ void store_rows(EncodeLds& L, const RowRegs& R, int lane) {
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int idx = k * 64 + lane, row = idx >> 4, c16 = idx & 15;
+    *reinterpret_cast<u32x4*>(&L.x[row * XROW + c16 * 8]) = R.v[k];
+  }
+}
+// Stage 16 rows into lds.x
+__device__ __forceinline__ void stage_rows(EncodeLds& L, const u16* __restrict__ src, long row_stride, int nvalid, int lane) {
+  RowRegs R;
+  load_rows(R, src, row_stride, nvalid, lane);
+  store_rows(L, R, lane);
 }
 __device__ __forceinline__ void stage_bases(EncodeLds& L, const uint8_t* __restrict__ b3row, const uint8_t* __restrict__ b4row, int lane) {
   if (lane < 32) reinterpret_cast<u32*>(L.b3)[lane] = reinterpret_cast<const u32*>(b3row)[lane];
@@ -37,41 +51,78 @@ __device__ __forceinline__ void wave_lds_sync() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier(); __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
+// The encoder works on 32-bit words that hold elements i and i+4 of a unit in their 16-bit halves (the decoder's word order), two
+// elements per VALU operation.
+struct BaseRegs { u32 b3[4][4], b4[4][4]; };      // [unit][i]: base of element i | base of element i+4 << 16
+template <int KIND>
+__device__ __forceinline__ void load_base_regs(const EncodeLds& L, int a, int q, BaseRegs& B) {
+#pragma unroll
+  for (int u = 0; u < 4; ++u) {
+    const int grp = unit_group<KIND>(a, q, u);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c0 = chan_of<KIND>(8 * grp + i), c1 = chan_of<KIND>(8 * grp + i + 4);
+      B.b3[u][i] = (u32)L.b3[c0] | ((u32)L.b3[c1] << 16);
+      B.b4[u][i] = (u32)L.b4[c0] | ((u32)L.b4[c1] << 16);
+    }
+  }
+}
+// the four data words of unit u of lane (a, q)
+template <int KIND>
+__device__ __forceinline__ void unit_data_words(const EncodeLds& L, int a, int q, int u, u32* __restrict__ W) {
+  if (KIND == KIND_K) {
+    // elements (2m, 2m+1) are the adjacent channels 32u + 2q + 8m (+1): four aligned words, re-paired to (i, i+4)
+    const u32* xr = reinterpret_cast<const u32*>(&L.x[a * XROW + 32 * u + 2 * q]);
+    const u32 r0 = xr[0], r1 = xr[4], r2 = xr[8], r3 = xr[12];
+    W[0] = __builtin_amdgcn_perm(r2, r0, 0x05040100u); W[1] = __builtin_amdgcn_perm(r2, r0, 0x07060302u);
+    W[2] = __builtin_amdgcn_perm(r3, r1, 0x05040100u); W[3] = __builtin_amdgcn_perm(r3, r1, 0x07060302u);
+  } else {
+    // element i is channel 64 (a & 1) + (a >> 1) + 8 i of token 4q + u
+    const u16* xr = &L.x[(4 * q + u) * XROW + 64 * (a & 1) + (a >> 1)];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) W[i] = (u32)xr[8 * i] | ((u32)xr[8 * i + 32] << 16);
+  }
+}
+typedef unsigned short u16x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ u32 pk_sub_u16(u32 x, u32 y) {
+  return __builtin_bit_cast(u32, (u16x2_t)(__builtin_bit_cast(u16x2_t, x) - __builtin_bit_cast(u16x2_t, y)));
+}
+
 // Encodes the tile staged in L (after a barrier).  Writes the native sign/mantissa and code bytes, the 16 tag words (one per line) and
 // the escape bytes (at esc_dst + offset-in-tile; nullptr = count only).  Returns the tile's escape byte count (all lanes).
-// Must be called by all 64 lanes of the wave that owns L; it synchronises that wave only.
+// Must be called by all 64 lanes of the wave that owns L; it synchronises that wave only.  B: load_base_regs of the same L.
 template <int KIND>
-__device__ __forceinline__ int encode_staged_tile(EncodeLds& L, int nvalid, int lane, uint8_t* __restrict__ sm_tile,
+__device__ __forceinline__ int encode_staged_tile(EncodeLds& L, const BaseRegs& B, int nvalid, int lane, uint8_t* __restrict__ sm_tile,
                                                   uint8_t* __restrict__ cd_tile, int* __restrict__ flags_tile,
                                                   uint8_t* __restrict__ esc_dst) {
   const int a = lane & 15, q = lane >> 4;
-  u32 slo[4], shi[4], g24[4], tag[4], eb[4];
-  u64 hi40[4];
+  u32 slo[4], shi[4], g24[4], tag[4], eb[4], ew[4][4];
 #pragma unroll
   for (int u = 0; u < 4; ++u) {
-    const int tok = unit_token<KIND>(a, q, u), grp = unit_group<KIND>(a, q, u);
-    bool fit3 = true, fit4 = true;
-    u32 c3 = 0, c4 = 0, cr = 0, s_lo = 0, s_hi = 0, e4 = 0;
-    u64 h = 0;
+    u32 W[4], d3[4], d4[4];
+    unit_data_words<KIND>(L, a, q, u, W);
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int ch = chan_of<KIND>(8 * grp + i);
-      const u32 x = L.x[tok * D + ch];
-      const int e = (int)((x >> 7) & 0xFFu);
-      const u32 smb = ((x >> 8) & 0x80u) | (x & 0x7Fu);
-      const int d3 = e - (int)L.b3[ch], d4 = e - (int)L.b4[ch];
-      fit3 = fit3 && ((unsigned)d3 < 8u);
-      fit4 = fit4 && ((unsigned)d4 < 16u);
-      c3 |= (u32)(d3 & 7) << (3 * i); c4 |= (u32)(d4 & 7) << (3 * i); cr |= (u32)(e & 7) << (3 * i);
-      e4 |= (u32)((d4 >> 3) & 1) << i;
-      h |= (u64)(e >> 3) << (5 * i);
-      if (i < 4) s_lo |= smb << (8 * i); else s_hi |= smb << (8 * (i - 4));
+    for (int i = 0; i < 4; ++i) {
+      ew[u][i] = (W[i] >> 7) & 0x00FF00FFu;                      // exponents
+      d3[i] = pk_sub_u16(ew[u][i], B.b3[u][i]); d4[i] = pk_sub_u16(ew[u][i], B.b4[u][i]);      // negative differences wrap to >= 0xFF01
     }
-    const bool valid = tok < nvalid;          // padded rows: tier 0, code 0, sign/mantissa 0
+    // tier rule (codec.py:144-150): all eight differences in 0..7, else all in 0..15, else raw
+    const bool fit3 = ((d3[0] | d3[1] | d3[2] | d3[3]) & 0xFFF8FFF8u) == 0u, fit4 = ((d4[0] | d4[1] | d4[2] | d4[3]) & 0xFFF0FFF0u) == 0u;
+    const bool valid = unit_token<KIND>(a, q, u) < nvalid;       // padded rows: tier 0, code 0, sign/mantissa 0
+    u32 cacc = 0u, xacc = 0u, sb[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const u32 c = fit3 ? d3[i] : (fit4 ? d4[i] : ew[u][i]);
+      cacc |= (c & 0x00070007u) << (3 * i);                       // code of element i at bits 3i, of element i+4 at 16 + 3i
+      xacc |= (d4[i] & 0x00080008u) << i;                         // 4th code bit of element i at bit 3 + i, of i+4 at 19 + i
+      sb[i] = ((W[i] >> 8) & 0x00800080u) | (W[i] & 0x007F007Fu); // sign/mantissa bytes at bits 0..7 and 16..23
+    }
+    const u32 p01 = __builtin_amdgcn_perm(sb[1], sb[0], 0x06020400u), p23 = __builtin_amdgcn_perm(sb[3], sb[2], 0x06020400u);
+    const u32 s_lo = __builtin_amdgcn_perm(p23, p01, 0x05040100u), s_hi = __builtin_amdgcn_perm(p23, p01, 0x07060302u);
     tag[u] = !valid || fit3 ? 0u : (fit4 ? 1u : 3u);
-    g24[u] = !valid ? 0u : (fit3 ? c3 : (fit4 ? c4 : cr));
+    g24[u] = valid ? (cacc & 0xFFFu) | ((cacc >> 16) << 12) : 0u;
     slo[u] = valid ? s_lo : 0u; shi[u] = valid ? s_hi : 0u;
-    eb[u] = e4; hi40[u] = h;
+    eb[u] = ((xacc >> 3) & 0xFu) | ((xacc >> 19) << 4);
   }
   // tag word of line a: this lane owns bits 8q..8q+7 (its four units)
   reinterpret_cast<uint8_t*>(L.tags)[4 * a + q] = (uint8_t)(tag[0] | (tag[1] << 2) | (tag[2] << 4) | (tag[3] << 6));
@@ -94,8 +145,13 @@ __device__ __forceinline__ int encode_staged_tile(EncodeLds& L, int nvalid, int 
     for (int u = 0; u < 4; ++u) {
       if (tag[u] == 1u) { p[0] = (uint8_t)eb[u]; p += 1; }
       else if (tag[u] == 3u) {
+        // raw group: the upper five exponent bits of the eight elements, 40 bits little-endian (element i at bit 5i)
+        u32 hl = 0u, hh = 0u;
 #pragma unroll
-        for (int k = 0; k < 5; ++k) p[k] = (uint8_t)(hi40[u] >> (8 * k));
+        for (int i = 0; i < 4; ++i) { hl |= ((ew[u][i] >> 3) & 0x1Fu) << (5 * i); hh |= ((ew[u][i] >> 19) & 0x1Fu) << (5 * i); }
+        const u64 h = (u64)hl | ((u64)hh << 20);
+#pragma unroll
+        for (int k = 0; k < 5; ++k) p[k] = (uint8_t)(h >> (8 * k));
         p += 5;
       }
     }
@@ -148,19 +204,22 @@ __device__ __forceinline__ void decode_tile_rows(const uint8_t* __restrict__ sm_
   }
 }
 
-// decode_tile_rows through an LDS staging tile (T*D u16, owned by the calling wave): the channel permutation turns the decoder's
-// output into 2-byte scattered stores, which LDS absorbs; global memory then gets 16-byte stores, a full 256-byte row per 16 lanes.
+// decode_tile_rows through an LDS staging tile (T rows of STAGE_ROW u16, owned by the calling wave): the channel permutation turns the
+// decoder's output into 2-byte scattered stores, which LDS absorbs; global memory then gets 16-byte stores, a full 256-byte row per
+// 16 lanes.  Rows are padded by 16 bytes: the sixteen lanes of a K line write sixteen different rows at the same column, which an
+// unpadded row stride (64 banks' worth) would send to one bank.
+constexpr int STAGE_ROW = D + 8;
 template <int KIND>
 __device__ __forceinline__ void decode_tile_staged(const uint8_t* __restrict__ sm_tile, const uint8_t* __restrict__ cd_tile,
                                                    const int* __restrict__ flags_tile, const uint8_t* __restrict__ esc,
                                                    const uint8_t* __restrict__ b3row, const uint8_t* __restrict__ b4row, int lane, int nvalid,
                                                    u16* __restrict__ stage, u16* __restrict__ out, long row_stride) {
-  decode_tile_rows<KIND>(sm_tile, cd_tile, flags_tile, esc, b3row, b4row, lane, T, stage, D);
+  decode_tile_rows<KIND>(sm_tile, cd_tile, flags_tile, esc, b3row, b4row, lane, T, stage, STAGE_ROW);
   wave_lds_sync();
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
     const int idx = k * 64 + lane, row = idx >> 4, c16 = idx & 15;
-    if (row < nvalid) *reinterpret_cast<u32x4*>(out + (long)row * row_stride + c16 * 8) = *reinterpret_cast<const u32x4*>(stage + row * D + c16 * 8);
+    if (row < nvalid) *reinterpret_cast<u32x4*>(out + (long)row * row_stride + c16 * 8) = *reinterpret_cast<const u32x4*>(stage + row * STAGE_ROW + c16 * 8);
   }
 }
 

@@ -55,14 +55,16 @@ __device__ __forceinline__ void store_tile(const PagedStoreArgs& A, EncodeLds& L
       u32x4 v = {0u, 0u, 0u, 0u};
       if (row >= off0) v = *reinterpret_cast<const u32x4*>(src + (long)(tok0 + row - off0) * stride + c16 * 8);
       else if (have) v = *reinterpret_cast<const u32x4*>(A.raw + ((long)r_old * T + row) * D + c16 * 8);
-      *reinterpret_cast<u32x4*>(&L.x[row * D + c16 * 8]) = v;
+      *reinterpret_cast<u32x4*>(&L.x[row * XROW + c16 * 8]) = v;
     }
     stage_bases(L, (KIND == KIND_K ? A.b3k : A.b3v) + (long)kvh * D, (KIND == KIND_K ? A.b4k : A.b4v) + (long)kvh * D, lane);
     wave_lds_sync();
+    BaseRegs Bs;
+    load_base_regs<KIND>(L, lane & 15, lane >> 4, Bs);
     uint8_t* slot = A.pool + p * A.TS;
-    const int total = encode_staged_tile<KIND>(L, T, lane, slot, slot + SLOT_CD, reinterpret_cast<int*>(slot + SLOT_FL), nullptr);
+    const int total = encode_staged_tile<KIND>(L, Bs, T, lane, slot, slot + SLOT_CD, reinterpret_cast<int*>(slot + SLOT_FL), nullptr);
     fits = total <= A.ovf_slot;
-    if (fits) encode_staged_tile<KIND>(L, T, lane, slot, slot + SLOT_CD, reinterpret_cast<int*>(slot + SLOT_FL), slot + SLOT_OV);
+    if (fits) encode_staged_tile<KIND>(L, Bs, T, lane, slot, slot + SLOT_CD, reinterpret_cast<int*>(slot + SLOT_FL), slot + SLOT_OV);
   }
   int r = r_old;
   if (!fits) {      // the rows stay raw: a filling block, or a finished tile whose escapes exceed the slot
@@ -130,7 +132,7 @@ __global__ void __launch_bounds__(64) k_paged_decode(const PagedDecodeArgs A) {
     return;
   }
   const uint8_t* slot = A.pool + (long)m * A.TS;
-  __shared__ __align__(16) u16 stage[T * D];
+  __shared__ __align__(16) u16 stage[T * STAGE_ROW];
   const bool aligned = (A.row_stride & 7) == 0 && (reinterpret_cast<uintptr_t>(out) & 15) == 0;
   if (kind) {
     if (aligned) decode_tile_staged<KIND_V>(slot, slot + SLOT_CD, reinterpret_cast<const int*>(slot + SLOT_FL), slot + SLOT_OV,

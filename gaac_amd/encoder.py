@@ -51,7 +51,7 @@ class TileEncoder:
     def compact(self, tile_bytes, head_start, ovf) -> torch.Tensor:
         """Pack the scratch slots into ovf at head_start[h] + tile_off[h, t]; returns tile_off int32 [H, ntiles]."""
         H, ntiles = tile_bytes.shape
-        tile_off = (torch.cumsum(tile_bytes, 1) - tile_bytes).to(torch.int32).contiguous()
+        tile_off = torch.empty_like(tile_bytes)
         _lib.call("gaac_compact", _lib.ptr(self._slots), _lib.ptr(tile_bytes), _lib.ptr(tile_off), _lib.ptr(head_start), _lib.ptr(ovf),
                   H, ntiles, _lib.stream())
         return tile_off

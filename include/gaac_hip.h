@@ -35,13 +35,15 @@ int gaac_encode_tiles(int kind, const void* x, int H, int S, int S_in, int S_pad
                       int n_kv, const int* bidx, uint8_t* sm, uint8_t* codes, int* flags, uint8_t* esc_slots, int* tile_bytes,
                       void* stream);
 
-/* TileEncoder.compact, /root/reference/gaac/encoder.py:69-76, 104-109: copies tile (h, t)'s tile_bytes[h, t] escape bytes
- * from its 1280-byte slot to ovf + head_start[h] + tile_off[h, t]. */
-int gaac_compact(const uint8_t* esc_slots, const int* tile_bytes, const int* tile_off, const int* head_start, uint8_t* ovf,
+/* TileEncoder.compact, /root/reference/gaac/encoder.py:69-76, 104-109: writes tile_off[h, t] = sum of tile_bytes[h, 0..t) (int32
+ * [H, ntiles], output) and copies tile (h, t)'s tile_bytes[h, t] escape bytes from its 1280-byte slot to
+ * ovf + head_start[h] + tile_off[h, t]. */
+int gaac_compact(const uint8_t* esc_slots, const int* tile_bytes, int* tile_off, const int* head_start, uint8_t* ovf,
                  int H, int ntiles, void* stream);
 
-/* row_offsets(flags, S), /root/reference/gaac/codec.py:221-225.  flags: int32 [H, S_pad]; out: int32 [H, S]. */
-int gaac_row_offsets(const int* flags, int H, int S, int S_pad, int* out, void* stream);
+/* row_offsets(flags, S), /root/reference/gaac/codec.py:221-225.  flags: int32 [H, S_pad]; out: int32 [H, S];
+ * chunk_sums: scratch, int32 [H * ceil(S / 2048)] (escape bytes per chunk of 2048 rows; written, then read). */
+int gaac_row_offsets(const int* flags, int H, int S, int S_pad, int* chunk_sums, int* out, void* stream);
 
 /* Codec.decode, /root/reference/gaac/codec.py:186-218.  Page fields as in the reference's Page dataclass
  * (codec.py:87-102) with tile_off [H, S_pad/16]; out: bf16, element (h, s, c) at out[h*out_head_stride + s*out_row_stride + c]. */
