@@ -260,7 +260,36 @@ def bench_codec(a):
     t0 = time.perf_counter()
     b3, b4 = O.calibrate(x16[:, :1024], 8); op = O.encode(x16, "k", b3, b4, 8); t1 = time.perf_counter(); od = O.decode(op); t2 = time.perf_counter()
     same = np.array_equal(od, x16) and int(op.ovf_head_start[-1]) == int(page.ovf_head_start[-1]) and np.array_equal(b3, codec.base3.cpu().numpy())
+    # the encoder and decoder kernels alone at the page size of config 1 (K and V [8, 65536, 128]), events around each launch, the
+    # inputs rotating over 3 copies; bytes = BF16 rows on one side + Page.nbytes on the other
+    from gaac_amd.codec import CB as _CB, row_offsets
+    full = {}
+    for kind, seed in (("k", 1), ("v", 2)):
+        x0 = make_kv(seed, N_KV, S_CTX).to(dev); xs = [x0, x0.clone(), x0.clone()]
+        c1 = Codec(N_KV).calibrate(x0[:, :1024]); e1 = TileEncoder(kind)
+        pgs = [e1.encode(c1, x0)]; pgs += [clone_store(pgs[0]), clone_store(pgs[0])]
+        smb = torch.empty(N_KV, S_CTX * D, dtype=torch.uint8, device=dev); cdb = torch.empty(N_KV, S_CTX * _CB, dtype=torch.uint8, device=dev)
+        flb = torch.zeros(N_KV, S_CTX, dtype=torch.int32, device=dev)
+        nb = x0.numel() * 2 + pgs[0].nbytes
+        def ev(fn, n=30):
+            for i in range(3): fn(i)
+            es = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(n)]
+            for i, (e0, e1_) in enumerate(es):
+                e0.record(); fn(i); e1_.record()
+            torch.cuda.synchronize()
+            return float(np.median([e0.elapsed_time(e1_) * 1e3 for e0, e1_ in es]))
+        te = ev(lambda i: e1.encode_tiles(xs[i % 3], c1.base3, c1.base4, smb, cdb, flb, S_CTX, S_CTX, N_KV))
+        tb = e1.encode_tiles(x0, c1.base3, c1.base4, smb, cdb, flb, S_CTX, S_CTX, N_KV)
+        ovf = torch.zeros_like(pgs[0].ovf)
+        tc = ev(lambda i: e1.compact(tb, pgs[0].ovf_head_start, ovf))
+        td = ev(lambda i: Codec.decode(pgs[i % 3]))
+        tr = ev(lambda i: row_offsets(pgs[i % 3].flags, S_CTX))
+        full[kind] = {"encode_tiles_us": round(te, 1), "encode_GBps": round(nb / te / 1e3, 1), "encode_frac_of_hbm_peak": round(nb / te / 1e3 / HBM_PEAK_GBS, 3),
+                      "compact_us": round(tc, 1), "decode_us": round(td, 1), "decode_GBps": round(nb / td / 1e3, 1),
+                      "decode_frac_of_hbm_peak": round(nb / td / 1e3 / HBM_PEAK_GBS, 3), "row_offsets_us": round(tr, 1), "bytes_in_plus_out": nb}
+        del xs, pgs, x0
     print(json.dumps({"workload": "config 0: codec round trip, K [8, 4096, 128] bf16", "ratio": round(page.ratio, 4), "tier_shares": [round(s3, 4), round(s4, 4), round(sr, 5)],
+                      "kernels_at_config1_page_size": full,
                       "bit_exact": exact, "matches_cpu_oracle": bool(same), "encode_us": round(t_enc, 1), "decode_us": round(t_dec, 1),
                       "encode_note": "TileEncoder.encode incl. its allocations and one host sync (sizes the escape stream)",
                       "cpu_oracle_encode_ms": round((t1 - t0) * 1e3, 1), "cpu_oracle_decode_ms": round((t2 - t1) * 1e3, 1)}))

@@ -13,7 +13,7 @@ P = c_void_p
 _SIGNATURES = {
     "gaac_exponent_hist": [P, c_long, c_int, P, P],
     "gaac_bases_from_hist": [P, c_int, P, P, P],
-    "gaac_encode_tiles": [c_int, P, c_int, c_int, c_int, c_int, P, P, c_int, P, P, P, P, P, P, P],
+    "gaac_encode_tiles": [c_int, P, c_long, c_long, c_int, c_int, c_int, P, P, c_int, P, P, P, P, P, P, P],
     "gaac_compact": [P, P, P, P, P, c_int, c_int, P],
     "gaac_row_offsets": [P, c_int, c_int, c_int, P, P, P],
     "gaac_decode_tiles": [c_int, P, P, P, P, P, P, P, P, c_int, P, c_int, c_int, c_int, P, c_long, c_long, P],

@@ -124,7 +124,7 @@ def encode_page(x: torch.Tensor, kind: str, base3: torch.Tensor, base4: torch.Te
     slots = scratch(H * ntiles * TILE_MAX_ESC, dev) if scratch else torch.empty(H * ntiles * TILE_MAX_ESC, dtype=torch.uint8, device=dev)
     tile_bytes = torch.empty(H, ntiles, dtype=torch.int32, device=dev)
     k = 0 if kind == "k" else 1
-    _lib.call("gaac_encode_tiles", k, _lib.ptr(x), H, S, S, S_pad, _lib.ptr(base3), _lib.ptr(base4), n_kv, None,
+    _lib.call("gaac_encode_tiles", k, _lib.ptr(x), S * D, D, H, S, S_pad, _lib.ptr(base3), _lib.ptr(base4), n_kv, None,
               _lib.ptr(sm), _lib.ptr(cd), _lib.ptr(flags), _lib.ptr(slots), _lib.ptr(tile_bytes), _lib.stream())
     head_bytes = tile_bytes.sum(1)
     head_start = torch.cat([torch.zeros(1, dtype=torch.int64, device=dev), torch.cumsum(head_bytes, 0)]).to(torch.int32).contiguous()

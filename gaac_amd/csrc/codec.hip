@@ -12,7 +12,10 @@ namespace gaac {
 char* last_error_buffer() { static thread_local char buf[512] = {0}; return buf; }
 
 // ---------------------------------------------------------------------------------------------------- calibration
-constexpr int HIST_CH = 32;     // channels per block (32 x 256 x 4 B = 32 KiB of LDS)
+// Exponent histogram per (kv head, channel).  A block owns 64 channels of the n_kv*128-wide token row and a chunk of tokens: eight
+// lanes read the 128 bytes of a row with 16-byte loads, counts go to LDS (64 x 256 x 4 B) and from there, where non-zero, to the
+// 64-bit global histogram.
+constexpr int HIST_CH = 64;
 __global__ void __launch_bounds__(256) k_exponent_hist(const u16* __restrict__ x, long n_tok, int n_kv, int chunk,
                                                        unsigned long long* __restrict__ hist) {
   __shared__ u32 h[HIST_CH * 256];
@@ -20,32 +23,58 @@ __global__ void __launch_bounds__(256) k_exponent_hist(const u16* __restrict__ x
   for (int i = tid; i < HIST_CH * 256; i += 256) h[i] = 0u;
   __syncthreads();
   const long t0 = (long)blockIdx.y * chunk, t1 = min(t0 + (long)chunk, n_tok);
-  const int c = tid & (HIST_CH - 1), sub = tid / HIST_CH;
+  const int c8 = tid & 7, sub = tid >> 3;
   const long row = (long)n_kv * D;
-  for (long t = t0 + sub; t < t1; t += 256 / HIST_CH) {
-    const u32 v = x[t * row + c0 + c];
-    atomicAdd(&h[c * 256 + ((v >> 7) & 0xFFu)], 1u);
+  const u16* xp = x + c0 + 8 * c8;
+  u32* hc = h + (8 * c8) * 256;
+  for (long t = t0 + sub; t < t1; t += 4 * 32) {      // four rows in flight per thread
+    u32x4 v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) v[k] = t + 32 * k < t1 ? *reinterpret_cast<const u32x4*>(xp + (t + 32 * k) * row) : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      if (t + 32 * k >= t1) break;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        atomicAdd(&hc[(2 * j) * 256 + ((v[k][j] >> 7) & 0xFFu)], 1u);
+        atomicAdd(&hc[(2 * j + 1) * 256 + ((v[k][j] >> 23) & 0xFFu)], 1u);
+      }
+    }
   }
   __syncthreads();
   for (int i = tid; i < HIST_CH * 256; i += 256)
     if (h[i]) atomicAdd(&hist[(long)(c0 + (i >> 8)) * 256 + (i & 255)], (unsigned long long)h[i]);
 }
 
-__global__ void __launch_bounds__(128) k_bases_from_hist(const long long* __restrict__ hist, int rows,
+// One wave per histogram row: lane l evaluates the windows that start at 4l .. 4l+3 (the reference takes the first maximum of the
+// window sums, codec.py:70-77: the lowest start wins ties).
+__global__ void __launch_bounds__(256) k_bases_from_hist(const long long* __restrict__ hist, int rows,
                                                          uint8_t* __restrict__ base3, uint8_t* __restrict__ base4) {
-  const int r = blockIdx.x * 128 + threadIdx.x;
+  __shared__ long long hs[4][256 + 16];
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = blockIdx.x * 4 + wave;
   if (r >= rows) return;
-  const long long* h = hist + (long)r * 256;
-  for (int pass = 0; pass < 2; ++pass) {          // densest 8-wide / 16-wide window, lowest start wins ties
+  long long* hr = hs[wave];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) hr[lane + 64 * k] = hist[(long)r * 256 + lane + 64 * k];
+  if (lane < 16) hr[256 + lane] = 0;
+  wave_lds_sync();
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
     const int w = pass ? 16 : 8;
-    long long s = 0;
-    for (int i = 0; i < w; ++i) s += h[i];
-    long long best = s; int arg = 0;
-    for (int st = 1; st + w <= 256; ++st) {
-      s += h[st + w - 1] - h[st - 1];
-      if (s > best) { best = s; arg = st; }
+    long long best = -1; int arg = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int st = 4 * lane + j;
+      long long sum = 0;
+      for (int i = 0; i < w; ++i) sum += hr[st + i];
+      if (st + w <= 256 && sum > best) { best = sum; arg = st; }
     }
-    (pass ? base4 : base3)[r] = (uint8_t)arg;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {      // maximum, lowest start among equals
+      const long long ob = __shfl_xor(best, o, 64); const int oa = __shfl_xor(arg, o, 64);
+      if (ob > best || (ob == best && oa < arg)) { best = ob; arg = oa; }
+    }
+    if (lane == 0) (pass ? base4 : base3)[r] = (uint8_t)arg;
   }
 }
 
@@ -55,7 +84,7 @@ __global__ void __launch_bounds__(128) k_bases_from_hist(const long long* __rest
 // registers while it encodes the current one.
 constexpr int CODEC_WAVES = 4, CODEC_TPW = 4, CODEC_TPB = CODEC_WAVES * CODEC_TPW;
 template <int KIND>
-__global__ void __launch_bounds__(64 * CODEC_WAVES) k_encode_tiles(const u16* __restrict__ x, int S, int S_in, int S_pad,
+__global__ void __launch_bounds__(64 * CODEC_WAVES) k_encode_tiles(const u16* __restrict__ x, int S, long x_head_stride, long x_row_stride, int S_pad,
                                                                    const uint8_t* __restrict__ base3, const uint8_t* __restrict__ base4,
                                                                    int n_kv, const int* __restrict__ bidx, uint8_t* __restrict__ sm,
                                                                    uint8_t* __restrict__ cd, int* __restrict__ flags,
@@ -66,9 +95,9 @@ __global__ void __launch_bounds__(64 * CODEC_WAVES) k_encode_tiles(const u16* __
   const int brow = bidx ? bidx[h] : h % n_kv;
   int tile = blockIdx.x * CODEC_TPB + wave;
   if (tile >= ntiles) return;
-  const u16* xh = x + (long)h * S_in * D;
+  const u16* xh = x + (long)h * x_head_stride;
   RowRegs R, Rn;
-  load_rows(R, xh + (long)tile * T * D, D, min(T, S - tile * T), lane);
+  load_rows(R, xh + (long)tile * T * x_row_stride, x_row_stride, min(T, S - tile * T), lane);
   stage_bases(L, base3 + (long)brow * D, base4 + (long)brow * D, lane);
   wave_lds_sync();
   BaseRegs Bs;                // the base words of the lane's units: the same for every tile of the head
@@ -76,7 +105,7 @@ __global__ void __launch_bounds__(64 * CODEC_WAVES) k_encode_tiles(const u16* __
   for (int i = 0; i < CODEC_TPW && tile < ntiles; ++i, tile += CODEC_WAVES) {
     const int nvalid = min(T, S - tile * T), next = tile + CODEC_WAVES;
     store_rows(L, R, lane);
-    if (i + 1 < CODEC_TPW && next < ntiles) load_rows(Rn, xh + (long)next * T * D, D, min(T, S - next * T), lane);
+    if (i + 1 < CODEC_TPW && next < ntiles) load_rows(Rn, xh + (long)next * T * x_row_stride, x_row_stride, min(T, S - next * T), lane);
     wave_lds_sync();
     const long row0 = (long)h * S_pad + (long)tile * T;
     const int total = encode_staged_tile<KIND>(L, Bs, nvalid, lane, sm + row0 * D, cd + row0 * CB, flags + row0,
@@ -212,7 +241,7 @@ const char* gaac_last_error(void) { return last_error_buffer(); }
 int gaac_exponent_hist(const void* x, long n_tokens, int n_kv, long long* hist, void* stream) {
   GAAC_REQUIRE(x && hist && n_kv > 0 && n_tokens >= 0, "gaac_exponent_hist: bad arguments");
   if (n_tokens == 0) return 0;
-  int nchunk = (int)min((n_tokens + 2047) / 2048, 256L);
+  int nchunk = (int)min((n_tokens + 1023) / 1024, 512L);
   int chunk = (int)((n_tokens + nchunk - 1) / nchunk);
   hipLaunchKernelGGL(k_exponent_hist, dim3(n_kv * D / HIST_CH, nchunk), dim3(256), 0, (hipStream_t)stream,
                      (const u16*)x, n_tokens, n_kv, chunk, (unsigned long long*)hist);
@@ -221,21 +250,23 @@ int gaac_exponent_hist(const void* x, long n_tokens, int n_kv, long long* hist, 
 
 int gaac_bases_from_hist(const long long* hist, int rows, uint8_t* base3, uint8_t* base4, void* stream) {
   GAAC_REQUIRE(hist && base3 && base4 && rows > 0, "gaac_bases_from_hist: bad arguments");
-  hipLaunchKernelGGL(k_bases_from_hist, dim3((rows + 127) / 128), dim3(128), 0, (hipStream_t)stream, hist, rows, base3, base4);
+  hipLaunchKernelGGL(k_bases_from_hist, dim3((rows + 3) / 4), dim3(256), 0, (hipStream_t)stream, hist, rows, base3, base4);
   return launch_status("gaac_bases_from_hist");
 }
 
-int gaac_encode_tiles(int kind, const void* x, int H, int S, int S_in, int S_pad, const uint8_t* base3, const uint8_t* base4,
-                      int n_kv, const int* bidx, uint8_t* sm, uint8_t* codes, int* flags, uint8_t* esc_slots, int* tile_bytes,
-                      void* stream) {
+int gaac_encode_tiles(int kind, const void* x, long x_head_stride, long x_row_stride, int H, int S, int S_pad, const uint8_t* base3,
+                      const uint8_t* base4, int n_kv, const int* bidx, uint8_t* sm, uint8_t* codes, int* flags, uint8_t* esc_slots,
+                      int* tile_bytes, void* stream) {
   GAAC_REQUIRE(kind == 0 || kind == 1, "gaac_encode_tiles: kind must be 0 (k) or 1 (v)");
   GAAC_REQUIRE(x && base3 && base4 && sm && codes && flags && esc_slots && tile_bytes, "gaac_encode_tiles: null pointer");
-  GAAC_REQUIRE(H > 0 && S > 0 && S_in >= S && S_pad >= (S + T - 1) / T * T && S_pad % T == 0 && n_kv > 0,
-               "gaac_encode_tiles: bad sizes H=%d S=%d S_in=%d S_pad=%d n_kv=%d", H, S, S_in, S_pad, n_kv);
+  GAAC_REQUIRE(H > 0 && S > 0 && S_pad >= (S + T - 1) / T * T && S_pad % T == 0 && n_kv > 0,
+               "gaac_encode_tiles: bad sizes H=%d S=%d S_pad=%d n_kv=%d", H, S, S_pad, n_kv);
+  GAAC_REQUIRE(x_row_stride >= D && x_row_stride % 8 == 0 && x_head_stride % 8 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0,
+               "gaac_encode_tiles: rows must be 16-byte aligned (strides in elements: head %ld, row %ld)", x_head_stride, x_row_stride);
   const int ntiles = (S + T - 1) / T;
   dim3 grid((ntiles + CODEC_TPB - 1) / CODEC_TPB, H);
-  if (kind == 0) hipLaunchKernelGGL(k_encode_tiles<KIND_K>, grid, dim3(64 * CODEC_WAVES), 0, (hipStream_t)stream, (const u16*)x, S, S_in, S_pad, base3, base4, n_kv, bidx, sm, codes, flags, esc_slots, tile_bytes, ntiles);
-  else hipLaunchKernelGGL(k_encode_tiles<KIND_V>, grid, dim3(64 * CODEC_WAVES), 0, (hipStream_t)stream, (const u16*)x, S, S_in, S_pad, base3, base4, n_kv, bidx, sm, codes, flags, esc_slots, tile_bytes, ntiles);
+  if (kind == 0) hipLaunchKernelGGL(k_encode_tiles<KIND_K>, grid, dim3(64 * CODEC_WAVES), 0, (hipStream_t)stream, (const u16*)x, S, x_head_stride, x_row_stride, S_pad, base3, base4, n_kv, bidx, sm, codes, flags, esc_slots, tile_bytes, ntiles);
+  else hipLaunchKernelGGL(k_encode_tiles<KIND_V>, grid, dim3(64 * CODEC_WAVES), 0, (hipStream_t)stream, (const u16*)x, S, x_head_stride, x_row_stride, S_pad, base3, base4, n_kv, bidx, sm, codes, flags, esc_slots, tile_bytes, ntiles);
   return launch_status("gaac_encode_tiles");
 }
 

@@ -38,13 +38,14 @@ class TileEncoder:
         return self._slots
 
     def encode_tiles(self, x, base3, base4, sm, cd, flags, S, S_pad, n_kv, bidx=None) -> torch.Tensor:
-        """Encode x [H, S_in, D] (tiles 0..ceil(S/16)-1) into sm/cd/flags with token stride S_pad; escape bytes stay in the
+        """Encode x [H, S_in, D] (any head / token strides, e.g. a transposed view of a token-major prompt; tiles 0..ceil(S/16)-1) into sm/cd/flags with token stride S_pad; escape bytes stay in the
         scratch slots.  Returns tile_bytes int32 [H, ntiles]; finish with compact()."""
         H = x.shape[0]; ntiles = (S + T - 1) // T; dev = x.device
-        x = x.contiguous()
+        if x.stride(2) != 1 or x.stride(0) % 8 or x.stride(1) % 8 or x.data_ptr() % 16:      # any head / row strides with 16-byte aligned rows
+            x = x.contiguous()
         slots = self._scratch(H * ntiles * SLOT, dev)
         tile_bytes = torch.empty(H, ntiles, dtype=torch.int32, device=dev)
-        _lib.call("gaac_encode_tiles", 0 if self.kind == "k" else 1, _lib.ptr(x), H, S, x.shape[1], S_pad, _lib.ptr(base3), _lib.ptr(base4),
+        _lib.call("gaac_encode_tiles", 0 if self.kind == "k" else 1, _lib.ptr(x), x.stride(0), x.stride(1), H, S, S_pad, _lib.ptr(base3), _lib.ptr(base4),
                   n_kv, _lib.ptr(bidx), _lib.ptr(sm), _lib.ptr(cd), _lib.ptr(flags), _lib.ptr(slots), _lib.ptr(tile_bytes), _lib.stream())
         return tile_bytes
 

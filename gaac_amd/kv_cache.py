@@ -55,7 +55,7 @@ class _Store:
                     self.head_start[h0:h1 + 1], self.tile_off[h0:h1], b3, b4, h1 - h0, S, n_kv, self.kind)
 
     def load_prompt(self, h0: int, h1: int, xh: torch.Tensor, n_kv: int, calibrate: bool, grow) -> None:
-        """xh: [n_kv, L, D].  Full tiles are compressed into rows [0, L//16*16) of the heads, the rest becomes the tail."""
+        """xh: [n_kv, L, D] (any strides).  Full tiles are compressed into rows [0, L//16*16) of the heads, the rest becomes the tail."""
         L = xh.shape[1]; full = L // T * T
         if calibrate:
             c = Codec(n_kv, xh.device).calibrate(xh)
@@ -115,7 +115,7 @@ class CompressedKVCache:
         assert L <= self.cap, f"sequence of {L} tokens exceeds the cache capacity {self.cap}"
         h0, h1 = slot * self.n_kv, (slot + 1) * self.n_kv
         for st, x in ((self.k, k), (self.v, v)):
-            st.load_prompt(h0, h1, x.transpose(0, 1).contiguous(), self.n_kv, self.per_sequence_bases, self._grow)
+            st.load_prompt(h0, h1, x.contiguous().transpose(0, 1), self.n_kv, self.per_sequence_bases, self._grow)      # a view: no transposing copy
         self.S[h0:h1] = L // T * T
         self.tail_len[h0:h1] = L % T
 

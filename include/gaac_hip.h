@@ -28,12 +28,13 @@ int gaac_exponent_hist(const void* x, long n_tokens, int n_kv, long long* hist, 
 int gaac_bases_from_hist(const long long* hist, int rows, uint8_t* base3, uint8_t* base4, void* stream);
 
 /* TileEncoder.encode_tiles, /root/reference/gaac/encoder.py:16-66, 94-102 (same math as Codec.encode, codec.py:133-184).
- * x: bf16 [H, S_in, 128]; tiles 0..ceil(S/16)-1 of every head are written to sm [H, S_pad*128], codes [H, S_pad*48],
- * flags [H, S_pad]; escape bytes of tile (h, t) go to esc_slots[(h*ntiles+t)*1280 ...]; tile_bytes: int32 [H, ntiles].
- * Head h uses base row bidx[h] (bidx != NULL) or h % n_kv. */
-int gaac_encode_tiles(int kind, const void* x, int H, int S, int S_in, int S_pad, const uint8_t* base3, const uint8_t* base4,
-                      int n_kv, const int* bidx, uint8_t* sm, uint8_t* codes, int* flags, uint8_t* esc_slots, int* tile_bytes,
-                      void* stream);
+ * x: bf16, element (h, s, c) at x[h*x_head_stride + s*x_row_stride + c] (head-major [H, S_in, 128] or a token-major prompt
+ * [S_in, H, 128] without a transposing copy; rows 16-byte aligned); tiles 0..ceil(S/16)-1 of every head are written to
+ * sm [H, S_pad*128], codes [H, S_pad*48], flags [H, S_pad]; escape bytes of tile (h, t) go to esc_slots[(h*ntiles+t)*1280 ...];
+ * tile_bytes: int32 [H, ntiles].  Head h uses base row bidx[h] (bidx != NULL) or h % n_kv. */
+int gaac_encode_tiles(int kind, const void* x, long x_head_stride, long x_row_stride, int H, int S, int S_pad, const uint8_t* base3,
+                      const uint8_t* base4, int n_kv, const int* bidx, uint8_t* sm, uint8_t* codes, int* flags, uint8_t* esc_slots,
+                      int* tile_bytes, void* stream);
 
 /* TileEncoder.compact, /root/reference/gaac/encoder.py:69-76, 104-109: writes tile_off[h, t] = sum of tile_bytes[h, 0..t) (int32
  * [H, ntiles], output) and copies tile (h, t)'s tile_bytes[h, t] escape bytes from its 1280-byte slot to
