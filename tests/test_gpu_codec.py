@@ -106,6 +106,52 @@ def test_row_offsets_matches_oracle():
     assert np.array_equal(got.cpu().numpy(), O.row_offsets(flags, 690))
 
 
+def test_row_offsets_over_many_chunks_and_a_ragged_end():
+    """The two-pass scan: several 2048-row chunks per head, a last chunk that is partly filled, S < S_pad."""
+    dev = require_gpu()
+    from gaac_amd.codec import row_offsets
+    rng = np.random.default_rng(4)
+    for S_pad, S in ((2048 * 3 + 16, 2048 * 3 + 5), (2048, 2048), (4096 + 2048, 4097)):
+        tags = rng.choice([0, 1, 3], size=(2, S_pad, 16), p=[0.7, 0.2, 0.1]).astype(np.int64)
+        flags = (tags << (2 * np.arange(16))).sum(-1).astype(np.uint32).view(np.int32)
+        got = row_offsets(torch.from_numpy(flags).to(dev), S)
+        assert np.array_equal(got.cpu().numpy(), O.row_offsets(flags, S)), (S_pad, S)
+
+
+def test_histogram_over_several_token_chunks():
+    """More tokens than one block's chunk, a token count that no loop stride divides, every exponent value present."""
+    dev = require_gpu()
+    from gaac_amd.codec import exponent_hist
+    n_kv, n_tok = 2, 5000 + 77
+    rng = np.random.default_rng(5)
+    x16 = rng.integers(0, 1 << 16, (n_tok, n_kv, 128), dtype=np.uint16)
+    hist = exponent_hist(to_bf16(x16, dev), n_kv)
+    assert np.array_equal(hist.cpu().numpy(), O.exponent_hist(x16, n_kv))
+    assert int(hist.sum()) == n_tok * n_kv * 128
+
+
+@pytest.mark.parametrize("kind", ["k", "v"])
+def test_encoder_reads_a_token_major_prompt_through_strides(kind):
+    """encode_tiles takes head and row strides: a transposed view of [L, n_kv, 128] encodes like its head-major copy; the page spans
+    several 16-tile blocks of the encoder with a partly filled last block and a partly filled last tile."""
+    dev = require_gpu()
+    from gaac_amd import Codec, TileEncoder
+    n_kv, L = 3, 16 * 37 + 9
+    x16 = kv_like16(n_kv, L, seed=21)
+    tm = to_bf16(np.ascontiguousarray(x16.transpose(1, 0, 2)), dev)          # [L, n_kv, 128]
+    view = tm.transpose(0, 1)
+    assert not view.is_contiguous()
+    codec = Codec(n_kv).calibrate(view[:, :200])
+    b3, b4 = O.calibrate(x16[:, :200], n_kv)
+    assert np.array_equal(codec.base3.cpu().numpy(), b3)
+    enc = TileEncoder(kind)
+    page_v, page_c = enc.encode(codec, view), enc.encode(codec, view.contiguous())
+    for f in ("sm", "codes", "flags", "ovf_off", "ovf", "ovf_head_start", "tile_off"):
+        assert torch.equal(getattr(page_v, f), getattr(page_c, f)), f
+    assert_pages_equal(native_to_reference_page(page_v), O.encode(x16, kind, b3, b4, n_kv))
+    assert np.array_equal(to_u16(Codec.decode(page_v)), x16)
+
+
 def test_base_collector_accumulates_over_steps_and_round_trips_its_file(tmp_path):
     """BaseCollector (calibration.py of the reference): histograms add up over prefill steps; bases equal the oracle's on the
     concatenated tokens; the saved file holds {layer: {k3,k4,v3,v4}} uint8 [n_kv,128] CPU tables and loads with weights_only."""
