@@ -320,8 +320,8 @@ def bench_paged(a):
     cal_k, cal_v = rows(1024, sig_k), rows(1024, sig_v)
     k3, k4 = bases_from_hist(exponent_hist(cal_k, n_kv), n_kv); v3, v4 = bases_from_hist(exponent_hist(cal_v, n_kv), n_kv)
     raw_tiles = 2 * n_kv * 4 * n_seq + need_blocks * 2 * n_kv // 100 + 64
-    st = LayerState(need_blocks, n_kv, raw_tiles, dict(k3=k3, k4=k4, v3=v3, v4=v4), 128, dev)
-    buf = torch.zeros(LayerState.pool_bytes(need_blocks, n_kv), dtype=torch.uint8, device=dev)
+    st = LayerState(need_blocks, n_kv, raw_tiles, dict(k3=k3, k4=k4, v3=v3, v4=v4), int(os.environ.get("GAAC_OVF_SLOT", 128)), dev)
+    buf = torch.zeros(LayerState.pool_bytes(need_blocks, n_kv, int(os.environ.get("GAAC_OVF_SLOT", 128))), dtype=torch.uint8, device=dev)
     for i, L in enumerate(lens):      # prompts
         ent = build_store_entries([0], [L], [bt_cpu[i]])
         st.store(rows(L, sig_k), rows(L, sig_v), buf, torch.from_numpy(ent).to(dev))
