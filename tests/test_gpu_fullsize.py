@@ -1,0 +1,95 @@
+"""Properties that hold at any size, checked at the full size of the headline configuration (batch 1, 32 q / 8 kv heads, d = 128,
+65536 compressed tokens + a 7-token tail), where the CPU oracle would take minutes: the round trip is the identity, the result does
+not depend on how the sequence is split, equal value rows come back unchanged, a zero query averages the values, and dropping the
+tail rows gives the attention over the compressed rows alone."""
+import numpy as np
+import pytest
+import torch
+
+from gpu_util import require_gpu
+
+pytestmark = pytest.mark.gpu
+N_KV, G, D, S, TAIL = 8, 4, 128, 65536, 7
+SCALE = D ** -0.5
+
+
+def _kv(seed, dev, spread):
+    """bf16 [N_KV, S + TAIL, D] made on the device: per-channel scales over `spread` octaves, sparse large values (all three tiers)."""
+    g = torch.Generator(device=dev).manual_seed(seed)
+    sig = torch.exp2(torch.rand(N_KV, 1, D, generator=g, device=dev) * spread - spread / 2)
+    x = torch.randn(N_KV, S + TAIL, D, generator=g, device=dev) * sig
+    hit = torch.rand(N_KV, S + TAIL, D, generator=g, device=dev) < 0.0003
+    return torch.where(hit, x * 4096.0, x).to(torch.bfloat16)
+
+
+def _encode(x, kind):
+    from gaac_amd import Codec, TileEncoder
+    c = Codec(N_KV).calibrate(x[:, :1024])
+    return TileEncoder(kind).encode(c, x[:, :S].contiguous())
+
+
+def _attend(q, kp, vp, k, v, nsplit, with_tail=True):
+    """the fused launch over the compressed pages (+ the raw tail rows S .. S+TAIL)"""
+    from gaac_amd.kernel import attn_launch
+    dev = q.device
+    kt = torch.zeros(N_KV, 16, D, dtype=torch.bfloat16, device=dev); vt = torch.zeros_like(kt)
+    kt[:, :TAIL] = k[:, S:]; vt[:, :TAIL] = v[:, S:]
+    TL = torch.full((N_KV,), TAIL if with_tail else 0, dtype=torch.int32, device=dev)
+    SL = torch.full((N_KV,), S, dtype=torch.int32, device=dev)
+    slots = torch.zeros(1, dtype=torch.int32, device=dev)
+    return attn_launch(kp, vp, q.reshape(N_KV * G, D), slots, N_KV * G, N_KV, SL, S, SCALE, nsplit, kt, vt, TL, 16).float()
+
+
+def _fp32_attention(q, k, v):
+    """textbook softmax attention in fp32 on the device over the given rows, GQA by repetition"""
+    qf = q.float().view(N_KV, G, D)
+    s = torch.einsum("hgd,hsd->hgs", qf, k.float()) * SCALE
+    return torch.einsum("hgs,hsd->hgd", torch.softmax(s, -1), v.float()).reshape(N_KV * G, D)
+
+
+def test_round_trip_is_the_identity_at_full_size():
+    dev = require_gpu()
+    from gaac_amd import Codec
+    for kind, seed in (("k", 1), ("v", 2)):
+        x = _kv(seed, dev, 8.0)[:, :S].contiguous()
+        page = _encode(x, kind)
+        assert torch.equal(Codec.decode(page).view(torch.int16), x.view(torch.int16))
+        assert 1.3 < page.ratio < 1.5
+        tags = page.flags.view(N_KV, S, 1) >> (2 * torch.arange(16, device=dev, dtype=torch.int32)) & 3
+        assert int((tags == 2).sum()) == 0 and int((tags == 1).sum()) > 0 and int((tags == 3).sum()) > 0      # tags are 0, 1 or 3
+
+
+def test_full_size_attention_properties():
+    dev = require_gpu()
+    k, v = _kv(11, dev, 2.0), _kv(12, dev, 2.0)
+    kp, vp = _encode(k, "k"), _encode(v, "v")
+    g = torch.Generator(device=dev).manual_seed(3)
+    q = (torch.randn(N_KV * G, D, generator=g, device=dev) * 0.3).to(torch.bfloat16)
+    ref = _fp32_attention(q, k, v)
+    mag = float(ref.abs().max())
+    outs = {n: _attend(q, kp, vp, k, v, n) for n in (1, 32, 61, 256)}
+    for n, o in outs.items():      # the reference's tolerance (tests/test_kernel.py:19) against fp32 attention over the same bf16 rows
+        assert float((o - ref).abs().max()) <= 2e-2 * mag + 1e-3, n
+    for n in (1, 61, 256):         # split-count independence up to fp32 summation order + the bf16 output rounding
+        assert float((outs[n] - outs[32]).abs().max()) <= 2.0 ** -7 * mag + 1e-6, n
+    # a zero query weighs every row alike: the output is the mean of the value rows
+    mean_v = v.float().mean(1, keepdim=True).expand(N_KV, G, D).reshape(N_KV * G, D)
+    o = _attend(torch.zeros_like(q), kp, vp, k, v, 32)
+    assert float((o - mean_v).abs().max()) <= 2e-2 * float(mean_v.abs().max()) + 1e-3
+    # without the tail rows the result is the attention over the compressed rows alone
+    o = _attend(q, kp, vp, k, v, 32, with_tail=False)
+    ref_c = _fp32_attention(q, k[:, :S], v[:, :S])
+    assert float((o - ref_c).abs().max()) <= 2e-2 * float(ref_c.abs().max()) + 1e-3
+
+
+def test_equal_value_rows_come_back_unchanged_at_full_size():
+    dev = require_gpu()
+    k = _kv(21, dev, 2.0)
+    row = (torch.randn(N_KV, 1, D, generator=torch.Generator(device=dev).manual_seed(5), device=dev) * 2).to(torch.bfloat16)
+    v = row.expand(N_KV, S + TAIL, D).contiguous()
+    kp, vp = _encode(k, "k"), _encode(v, "v")
+    q = torch.randn(N_KV * G, D, generator=torch.Generator(device=dev).manual_seed(6), device=dev).to(torch.bfloat16)
+    o = _attend(q, kp, vp, k, v, 32)
+    want = row.float().expand(N_KV, G, D).reshape(N_KV * G, D)
+    # softmax weights sum to one: every output row is the value row, up to the fp32 normalisation and the bf16 rounding of the output
+    assert float((o - want).abs().max()) <= 2.0 ** -7 * float(want.abs().max())
