@@ -164,13 +164,18 @@ __device__ __forceinline__ void raw_rows_attend(RawScratch& R, const u16* __rest
                                                 float (*__restrict__ acc5)[D]) {
   __syncthreads();               // qs is filled / the previous call is done with sc
   const int t = tid >> 4, c = tid & 15;
-  float kr[8];
-  {
-    u32x4 kv = {0u, 0u, 0u, 0u};
-    if (t < nvalid && t < T) kv = *reinterpret_cast<const u32x4*>(krows + t * D + 8 * c);
+  // all global loads of the call up front (one memory latency): this thread's piece of a K row, and for the output the two
+  // channels 2 (tid & 63), +1 of all 16 V rows
+  u32x4 kv = {0u, 0u, 0u, 0u};
+  if (t < nvalid && t < T) kv = *reinterpret_cast<const u32x4*>(krows + t * D + 8 * c);
+  u32 vv[T];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) { kr[2 * i] = bf16_bits_to_float(kv[i] & 0xFFFFu); kr[2 * i + 1] = bf16_bits_to_float(kv[i] >> 16); }
-  }
+  for (int tk = 0; tk < T; ++tk) vv[tk] = *reinterpret_cast<const u32*>(vrows + min(tk, max(nvalid - 1, 0)) * D + 2 * (tid & 63));
+#pragma unroll
+  for (int tk = 0; tk < T; ++tk) vv[tk] = tk < nvalid ? vv[tk] : 0u;      // rows past the end weigh 0: keep an Inf of the clamped row out of 0 * Inf
+  float kr[8];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) { kr[2 * i] = bf16_bits_to_float(kv[i] & 0xFFFFu); kr[2 * i + 1] = bf16_bits_to_float(kv[i] >> 16); }
   for (int g = 0; g < G; ++g) {
     float d = 0.f;
 #pragma unroll
@@ -187,7 +192,7 @@ __device__ __forceinline__ void raw_rows_attend(RawScratch& R, const u16* __rest
 #pragma unroll
     for (int o = 8; o > 0; o >>= 1) mt = fmaxf(mt, __shfl_xor(mt, o, 16));
     const float m_old = g < G ? m5[g] : -INFINITY, m_new = fmaxf(m_old, mt), mu = m_new == -INFINITY ? 0.f : m_new;
-    const float p = __builtin_amdgcn_exp2f(s - mu);
+    const float p = __builtin_amdgcn_exp2f(s - mu);        // rows >= nvalid: exp2(-inf) = 0
     float lt = p;
 #pragma unroll
     for (int o = 8; o > 0; o >>= 1) lt += __shfl_xor(lt, o, 16);
@@ -201,11 +206,13 @@ __device__ __forceinline__ void raw_rows_attend(RawScratch& R, const u16* __rest
     }
   }
   __syncthreads();
-  const int d = tid & 127;
-  for (int g = tid >> 7; g < G; g += NT / 128) {
-    float acc = acc5[g][d] * R.alpha[g];
-    for (int tk = 0; tk < nvalid; ++tk) acc += R.sc[g][tk] * bf16_bits_to_float(vrows[tk * D + d]);
-    acc5[g][d] = acc;
+  const int d2 = 2 * (tid & 63);
+  for (int g = tid >> 6; g < G; g += NT / 64) {
+    const float al = R.alpha[g];
+    float a0 = acc5[g][d2] * al, a1 = acc5[g][d2 + 1] * al;
+#pragma unroll
+    for (int tk = 0; tk < T; ++tk) { const float p = R.sc[g][tk]; a0 += p * bf16_bits_to_float(vv[tk] & 0xFFFFu); a1 += p * bf16_bits_to_float(vv[tk] >> 16); }
+    acc5[g][d2] = a0; acc5[g][d2 + 1] = a1;
   }
 }
 
@@ -567,8 +574,30 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
                  "s"(A.k.head_start), "s"(A.k.base3), "s"(A.k.base4), "s"(A.v.sm), "s"(A.v.cd), "s"(A.v.flags), "s"(A.v.tile_off),
                  "s"(A.v.ovf), "s"(A.v.head_start), "s"(A.v.base3), "s"(A.v.base4), "s"(A.kt), "s"(A.tl), "s"(A.nsplit), "s"(A.n_kv),
                  "s"(A.n_q), "s"(A.G), "s"(A.NB), "s"(A.S_pad), "s"(A.tcap));
-  const int bh = (int)blockIdx.x / A.nsplit, split = (int)blockIdx.x % A.nsplit;
-  const int b = bh / A.n_kv, kvh = bh % A.n_kv, G = A.G;
+  // Paged pool: the split index is rotated by the head index: the last split of a sequence carries the raw tile that is still filling,
+  // and with equal split counts all of them would otherwise sit on the same XCD, which then finishes long after the others.
+  const int bh = (int)blockIdx.x / A.nsplit, split = ((int)blockIdx.x + (PAGED ? bh : 0)) % A.nsplit;
+  int b = bh / A.n_kv, S_ranked = -1;
+  const int kvh = bh % A.n_kv, G = A.G;
+  if (PAGED) {
+    // Ragged batches: blocks start in index order, so the longest sequences go first and the short ones fill the end of the launch
+    // (in batch order a long sequence that happens to come last runs on with most of the GPU idle).  Batch row = the sequence whose
+    // length has rank b; every block ranks the lengths itself (thread i counts the sequences ahead of sequence i).
+    const int Bn = (int)gridDim.x / (A.nsplit * A.n_kv);
+    if (Bn > 1 && Bn <= NT) {
+      int* lens = reinterpret_cast<int*>(&M.acc[0][0][0]);      // the merge buffer is idle until the tile loop has ended
+      const int mine = tid < Bn ? max(A.sl[tid], 0) : 0;
+      if (tid < Bn) lens[tid] = mine;
+      __syncthreads();
+      if (tid < Bn) {
+        int rank = 0;
+        for (int j = 0; j < Bn; ++j) { const int lj = lens[j]; rank += (lj > mine || (lj == mine && j < tid)) ? 1 : 0; }
+        if (rank == b) { lens[NT] = tid; lens[NT + 1] = mine; }
+      }
+      __syncthreads();
+      b = __builtin_amdgcn_readfirstlane(lens[NT]); S_ranked = __builtin_amdgcn_readfirstlane(lens[NT + 1]);
+    }
+  }
   const long qh0 = (long)b * A.n_q + (long)kvh * G;
   // Level 1: the slot of the batch row; the query rows do not depend on it
   TableRegs Tr;
@@ -576,7 +605,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
   const int slot = PAGED ? 0 : A.slot[b], ch = PAGED ? kvh : (slot < 0 ? 0 : slot) * A.n_kv + kvh;
   // Level 2: everything indexed by the cache head
   int S, TLh = 0; long khs = 0, vhs = 0;
-  if (PAGED) S = max(A.sl[b], 0);
+  if (PAGED) S = S_ranked >= 0 ? S_ranked : max(A.sl[b], 0);
   else {
     S = A.sl[ch]; khs = A.k.head_start[ch]; vhs = A.v.head_start[ch];
     TLh = (A.kt ? A.tl : A.sl)[ch];            // no branch between the loads of this level
@@ -1022,7 +1051,7 @@ extern "C" int gaac_paged_attn(
   A.tickets = tickets; A.out = (u16*)out;
   A.pool = pool; A.raw = (const u16*)raw; A.mt = mt; A.bt = bt; A.bt_stride = bt_stride; A.TS = TS;
 #ifdef GAAC_PHASE_TIMING
-  A.dbg = nullptr;
+  A.dbg = g_dbg;
 #endif
   if ((long)B * n_kv * nsplit <= 256) hipLaunchKernelGGL((k_attn_split<true, 8>), dim3(B * n_kv * nsplit), dim3(512), 0, (hipStream_t)stream, A);
   else hipLaunchKernelGGL((k_attn_split<true, 4>), dim3(B * n_kv * nsplit), dim3(256), 0, (hipStream_t)stream, A);
