@@ -78,6 +78,7 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1); ap.add_argument("--steps", type=int, default=300); ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--copies", type=int, default=3); ap.add_argument("--nsplit", type=int, default=0)
+    ap.add_argument("--batch", type=int, default=1, help="decode64k only: batch rows (each with its own 65536-token context); the headline is 1")
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="also run the library's plain 64 MiB copy kernel 10 times (the known-size kernel for scaling FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--cpu-heads", type=int, default=8, help="kv heads in the CPU baseline sample (0 = skip)")
@@ -101,12 +102,13 @@ def main():
     from gaac_amd import Codec, TileEncoder
     from gaac_amd.kernel import attn_launch, choose_nsplit, AttnWorkspace
     dev = "cuda"
-    n_q, H = N_KV * G, N_KV
+    B = a.batch
+    n_q, H = N_KV * G, B * N_KV
     scale = D ** -0.5
 
     # ---- synthetic inputs (config 1): K seed 1, V seed 2, q seed 3; bases from the first 1024 tokens
     k_all, v_all = make_kv(1, H, S_CTX + TAIL_TOK), make_kv(2, H, S_CTX + TAIL_TOK, *v_range)
-    q = torch.randn(1, n_q, D, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
+    q = torch.randn(B, n_q, D, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
     kd, vd, qd = k_all.to(dev), v_all.to(dev), q.to(dev)
     ck, cv = Codec(N_KV).calibrate(kd[:, :1024]), Codec(N_KV).calibrate(vd[:, :1024])
     kp = TileEncoder("k").encode(ck, kd[:, :S_CTX].contiguous()); vp = TileEncoder("v").encode(cv, vd[:, :S_CTX].contiguous())
@@ -114,14 +116,14 @@ def main():
     kt[:, :TAIL_TOK] = kd[:, S_CTX:]; vt[:, :TAIL_TOK] = vd[:, S_CTX:]
     TL = torch.full((H,), TAIL_TOK, dtype=torch.int32, device=dev)
     SL = torch.full((H,), S_CTX, dtype=torch.int32, device=dev)
-    slots = torch.zeros(1, dtype=torch.int32, device=dev)
-    nsplit = a.nsplit or choose_nsplit(1, N_KV, S_CTX)
-    ws = AttnWorkspace(n_q, nsplit, torch.bfloat16, dev)
-    q2d = qd.reshape(n_q, D).contiguous()
+    slots = torch.arange(B, dtype=torch.int32, device=dev)
+    nsplit = a.nsplit or choose_nsplit(B, N_KV, S_CTX)
+    ws = AttnWorkspace(B * n_q, nsplit, torch.bfloat16, dev)
+    q2d = qd.reshape(B * n_q, D).contiguous()
     S_pad = kp.sm.shape[1] // D
     pages = [(kp, vp)] + [(clone_store(kp), clone_store(vp)) for _ in range(a.copies - 1)]
-    alg_bytes = kp.nbytes + vp.nbytes + 2 * N_KV * TAIL_TOK * D * 2 + 2 * n_q * D * 2 + 4 * N_KV * D
-    bf16_bytes = 2 * H * (S_CTX + TAIL_TOK) * D * 2 + 2 * n_q * D * 2
+    alg_bytes = kp.nbytes + vp.nbytes + 2 * H * TAIL_TOK * D * 2 + 2 * B * n_q * D * 2 + 4 * N_KV * D
+    bf16_bytes = 2 * H * (S_CTX + TAIL_TOK) * D * 2 + 2 * B * n_q * D * 2
 
     def step(i, phase="fused"):
         K, V = pages[i % len(pages)]
@@ -140,7 +142,7 @@ def main():
     kdec = torch.cat([Codec.decode(kp), kd[:, S_CTX:]], 1).float(); vdec = torch.cat([Codec.decode(vp), vd[:, S_CTX:]], 1).float()
     assert torch.equal(kdec[:, :S_CTX].to(torch.bfloat16).view(torch.int16), kd[:, :S_CTX].view(torch.int16)), "round trip is not bit-exact"
     sc = torch.einsum("hgd,hsd->hgs", q2d.float().view(H, G, D), kdec) * scale
-    ref = torch.einsum("hgs,hsd->hgd", torch.softmax(sc, -1), vdec).reshape(n_q, D)
+    ref = torch.einsum("hgs,hsd->hgd", torch.softmax(sc, -1), vdec).reshape(B * n_q, D)
     err_max, err_mean = (out - ref).abs().max().item(), (out - ref).abs().mean().item()
     del kdec, vdec, sc
 
@@ -180,12 +182,12 @@ def main():
     # (b) torch's scaled_dot_product_attention, for reference only
     from gaac_amd.kernel import bf16_attention
     kb = [kd.clone() for _ in range(a.copies)]; vb = [vd.clone() for _ in range(a.copies)]
-    qb = qd.view(1, n_q, D)
-    ref_b = bf16_attention(qb, kb[0], vb[0], scale).float().view(n_q, D)
+    qb = qd.view(B, n_q, D)
+    ref_b = bf16_attention(qb, kb[0], vb[0], scale).float().view(B * n_q, D)
     assert (ref_b - ref).abs().max().item() <= 1e-2, "baseline kernel is off"
     bf16_us, bf16_ns = None, None
-    for ns in (64, 96, 128, 192):
-        wsb = AttnWorkspace(n_q, ns, torch.bfloat16, dev)
+    for ns in sorted({max(1, x // B) for x in (64, 96, 128, 192)}):
+        wsb = AttnWorkspace(B * n_q, ns, torch.bfloat16, dev)
         for i in range(10): bf16_attention(qb, kb[i % a.copies], vb[i % a.copies], scale, ns, wsb)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         n_b = max(60, a.steps // 2)
@@ -194,8 +196,8 @@ def main():
         e1.record(); torch.cuda.synchronize()
         t = e0.elapsed_time(e1) * 1e3 / n_b
         if bf16_us is None or t < bf16_us: bf16_us, bf16_ns = t, ns
-    q4 = qd.view(1, n_q, 1, D)
-    k4 = [x.view(1, H, S_CTX + TAIL_TOK, D) for x in kb]; v4 = [x.view(1, H, S_CTX + TAIL_TOK, D) for x in vb]
+    q4 = qd.view(B, n_q, 1, D)
+    k4 = [x.view(B, N_KV, S_CTX + TAIL_TOK, D) for x in kb]; v4 = [x.view(B, N_KV, S_CTX + TAIL_TOK, D) for x in vb]
     sdpa = lambda i: torch.nn.functional.scaled_dot_product_attention(q4, k4[i % a.copies], v4[i % a.copies], scale=scale, enable_gqa=True)
     for i in range(3): sdpa(i)
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -206,10 +208,10 @@ def main():
 
     s3k, s4k, srk = tier_shares(kp); s3v, s4v, srv = tier_shares(vp)
     res = {
-        "metric": f"64K decode-attn us/layer + effective HBM GB/s (b=1, n_kv={N_KV}, g={G}, d=128)", "value": round(us_step, 3), "unit": "us/layer",
+        "metric": f"64K decode-attn us/layer + effective HBM GB/s (b={B}, n_kv={N_KV}, g={G}, d=128)", "value": round(us_step, 3), "unit": "us/layer",
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(us_step / 1e3, 6), "higher_is_better": False,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"config {1 if G == 4 else 2}: fused decode attention, batch 1, {n_q} q heads / {N_KV} kv heads, d=128, 65536 compressed tokens + 7-token bf16 tail",
+        "config": {"workload": f"config {1 if G == 4 else 2}: fused decode attention, batch {B}, {n_q} q heads / {N_KV} kv heads, d=128, 65536 compressed tokens + 7-token bf16 tail",
                    "nsplit": nsplit, "kv_copies_rotated": len(pages), "timing": "one HIP graph of all steps, wall clock between synchronizes"},
         "effective_GBps": round(alg_bytes / us_step / 1e3, 1), "algorithmic_bytes": alg_bytes, "bf16_bytes": bf16_bytes,
         "compression_ratio_k": round(kp.ratio, 4), "compression_ratio_v": round(vp.ratio, 4),
@@ -220,10 +222,10 @@ def main():
                           "torch_sdpa_us": round(sdpa_us, 1)},
         "roofline": {"bound": "hbm", "achieved": round(alg_bytes / split_us_mean / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(alg_bytes / split_us_mean / 1e3 / HBM_PEAK_GBS, 4),
-                     "traffic": MEASURED_TRAFFIC["bytes"] if nsplit == MEASURED_TRAFFIC["nsplit"] and a.workload == "decode64k" else None,
+                     "traffic": MEASURED_TRAFFIC["bytes"] if nsplit == MEASURED_TRAFFIC["nsplit"] and a.workload == "decode64k" and B == 1 else None,
                      "kernel": "k_attn_split (split pass + tail + fused merge)", "kernel_us_mean": round(split_us_mean, 2), "kernel_us_median": round(split_us_med, 2)},
     }
-    if a.cpu_heads > 0:
+    if a.cpu_heads > 0 and B == 1:
         b = lambda t: t.cpu().numpy()
         u16 = lambda t: t.contiguous().view(torch.int16).numpy().view(np.uint16)
         res["cpu_baseline"] = cpu_baseline(u16(k_all[:, :S_CTX]), u16(v_all[:, :S_CTX]), u16(q.view(n_q, D)), b(ck.base3), b(ck.base4), b(cv.base3), b(cv.base4), scale, a.cpu_heads)
