@@ -93,3 +93,35 @@ def test_equal_value_rows_come_back_unchanged_at_full_size():
     want = row.float().expand(N_KV, G, D).reshape(N_KV * G, D)
     # softmax weights sum to one: every output row is the value row, up to the fp32 normalisation and the bf16 rounding of the output
     assert float((o - want).abs().max()) <= 2.0 ** -7 * float(want.abs().max())
+
+
+def test_byte_offsets_beyond_4_gib():
+    """Five batch rows of 2^20 tokens: the sign/mantissa array of a page is 5 GiB, so the last row's tiles sit beyond 32-bit byte
+    offsets in every kernel (encoder, decoder, attention).  Checked on the first and the last row."""
+    dev = require_gpu()
+    from gaac_amd import Codec, TileEncoder, attention
+    B, n_kv, g_, S_ = 5, 8, 2, 1 << 20
+    gen = torch.Generator(device=dev).manual_seed(31)
+    def make(seed_shift):
+        sig = torch.exp2(torch.rand(B * n_kv, 1, D, generator=gen, device=dev) * 2 - 1)
+        x = torch.empty(B * n_kv, S_, D, dtype=torch.bfloat16, device=dev)
+        for h in range(B * n_kv):      # head by head: no fp32 copy of the whole tensor
+            x[h] = (torch.randn(S_, D, generator=gen, device=dev) * sig[h]).to(torch.bfloat16)
+        return x
+    k, v = make(0), make(1)
+    ck, cv = Codec(n_kv).calibrate(k[:n_kv, :2048]), Codec(n_kv).calibrate(v[:n_kv, :2048])
+    kp, vp = TileEncoder("k").encode(ck, k), TileEncoder("v").encode(cv, v)
+    assert kp.sm.numel() > (1 << 32) and kp.sm.shape == (B * n_kv, S_ * D)
+    for page, x in ((kp, k), (vp, v)):
+        back = Codec.decode(page)
+        for h in (0, B * n_kv - 1):
+            assert torch.equal(back[h].view(torch.int16), x[h].view(torch.int16)), h
+        del back
+    q = (torch.randn(B, n_kv * g_, D, generator=gen, device=dev) * 0.3).to(torch.bfloat16)
+    out = attention(q, kp, vp, SCALE).float()
+    for b in (0, B - 1):
+        kb, vb = k[b * n_kv:(b + 1) * n_kv].float(), v[b * n_kv:(b + 1) * n_kv].float()
+        s = torch.einsum("hgd,hsd->hgs", q[b].float().view(n_kv, g_, D), kb) * SCALE
+        ref = torch.einsum("hgs,hsd->hgd", torch.softmax(s, -1), vb).reshape(n_kv * g_, D)
+        assert float((out[b] - ref).abs().max()) <= 2e-2 * float(ref.abs().max()) + 1e-3, b
+        del kb, vb, s
