@@ -106,6 +106,22 @@ def test_prefill_then_decode_steps_through_a_permuted_block_table():
     P.check([0, 1, 2, 3], randn_bf16((4, N_KV * G, 128), seed=79, scale=0.1), nsplit=20)      # 320 blocks: the four-wave block shape
 
 
+def test_pool_beyond_4_gib_and_ragged_lengths_taken_longest_first():
+    """A slot pool of 4.8 GB: most of the permuted block table points beyond 32-bit byte offsets.  Six sequences of very different
+    lengths in an order that is neither ascending nor descending (the kernel takes them longest first; outputs stay in batch order)."""
+    dev = require_gpu()
+    P = _Pool(dev, n_seq=6, max_blocks=84, num_blocks=200_000, raw_tiles=128, seed=5)
+    assert P.buf.numel() > (1 << 32) and int(P.bt_cpu.max()) * 2 * N_KV * P.st.TS > (1 << 32)
+    lens = {0: 300, 1: 1270, 2: 16, 3: 777, 4: 1270, 5: 45}
+    P.step({s: _rows(n, 40 + s) for s, n in lens.items()})
+    P.check([0, 1, 2, 3, 4, 5], randn_bf16((6, N_KV * G, 128), seed=91, scale=0.1))
+    P.check([5, 3, 1], randn_bf16((3, N_KV * G, 128), seed=92, scale=0.1), nsplit=3)
+    for step in range(20):
+        P.step({s: _rows(1, 3000 + 11 * step + s) for s in range(6)})
+    P.check([2, 4, 0, 5, 1, 3], randn_bf16((6, N_KV * G, 128), seed=93, scale=0.1), nsplit=5)
+    P.st.check()
+
+
 def test_tiles_whose_escapes_do_not_fit_stay_raw_and_blocks_are_released():
     dev = require_gpu()
     P = _Pool(dev, n_seq=2, max_blocks=8, num_blocks=32, raw_tiles=72, ovf_slot=32)
