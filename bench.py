@@ -345,6 +345,12 @@ def bench_paged(a):
         torch.cuda.synchronize()
         t_store.append(e[0].elapsed_time(e[1]) * 1e3); t_attn.append(e[1].elapsed_time(e[2]) * 1e3)
     st.check()
+    # chunked-prefill support: decode the longest sequence's blocks into flat scratch K/V (bit-exact rows for a prefill attention)
+    li = int(np.argmax(cur)); nb_l = -(-cur[li] // BLOCK)
+    pairs = torch.tensor([(int(bt_cpu[li][j]), 16 * j, min(16, cur[li] - 16 * j)) for j in range(nb_l)], dtype=torch.int32, device=dev)
+    sk = torch.empty(cur[li], n_kv, D, dtype=torch.bfloat16, device=dev); sv = torch.empty_like(sk)
+    t_dec = _median_us(lambda: st.decode_blocks(buf, pairs, sk, sv), 20)
+    dec_bytes = nb_l * 2 * n_kv * 2880 + 2 * sk.numel() * 2
     # bytes the attention has to read: full slots up to the used escape bytes, raw tiles in full
     mt = st.mt.cpu().numpy().reshape(need_blocks, 2 * n_kv)
     n_tiles = sum(-(-c // BLOCK) for c in cur) * 2 * n_kv
@@ -359,7 +365,8 @@ def bench_paged(a):
                       "attention_us": round(med(t_attn), 1), "store_us": round(med(t_store), 1), "step_us": round(med(t_attn) + med(t_store), 1),
                       "attention_read_GBps": round(read_bytes / med(t_attn) / 1e3, 1), "bf16_equivalent_GBps": round(bf16_bytes / med(t_attn) / 1e3, 1),
                       "slot_pool_bytes": pool_bytes, "bf16_pool_bytes": bf16_pool, "pool_ratio": round(bf16_pool / pool_bytes, 4),
-                      "raw_tiles_in_use": n_raw, "tiles": n_tiles}))
+                      "raw_tiles_in_use": n_raw, "tiles": n_tiles,
+                      "decode_blocks": {"tokens": cur[li], "us": round(t_dec, 1), "GBps_in_plus_out": round(dec_bytes / t_dec / 1e3, 1)}}))
 
 
 def bench_serve(a):
