@@ -171,3 +171,43 @@ def test_other_head_shapes_with_random_batches(n_kv, G):
     for s in range(n_slots):
         dk, dv = cache.decompress(s)
         assert np.array_equal(to_u16(dk), hist[s][0]) and np.array_equal(to_u16(dv), hist[s][1])
+
+
+def test_many_rows_with_short_and_tail_only_sequences():
+    """A batch of 72 rows over 80 slots (more than 256 blocks: the four-wave block shape, one split per head): sequences of 1..70 tokens,
+    many of them shorter than one tile, so the only partial of a head is the one its first wave makes from the raw tail rows."""
+    dev = require_gpu()
+    from gaac_amd import CompressedKVCache
+    n_slots = 80
+    cache = CompressedKVCache(n_slots=n_slots, n_kv=N_KV, capacity=128, bases=_bases(12, dev))
+    rng = np.random.default_rng(8)
+    hist = {}
+    order = rng.permutation(n_slots)[:72]
+    for s in order:
+        L = int(rng.integers(1, 71)) if s % 5 else int(rng.integers(1, 16))
+        k16, v16 = _prompt(L, 900 + int(s))
+        cache.prefill(int(s), to_bf16(k16, dev), to_bf16(v16, dev)); hist[int(s)] = (k16, v16)
+    slots_l = [int(s) for s in order]
+    slots_l[5] = -1; slots_l[40] = -1
+    q16 = randn_bf16((72, N_KV * G, 128), seed=77, scale=0.1)
+    slots = torch.tensor(slots_l, dtype=torch.int32, device=dev)
+    out = O.bf16_to_f32(to_u16(cache.attention(to_bf16(q16, dev), slots, SCALE)))
+    for b, s in enumerate(slots_l):
+        if s < 0:
+            assert np.abs(out[b]).max() == 0
+            continue
+        ref = O.ref_attention(q16[b], hist[s][0], hist[s][1], SCALE)
+        assert np.abs(out[b] - ref).max() <= 2e-2 * np.abs(ref).max() + 1e-3, (b, s, len(hist[s][0]))
+    # one decode step on every live row, then the same check on a few rows
+    k16 = randn_bf16((72, N_KV, 128), seed=78, scale=0.5); v16 = randn_bf16((72, N_KV, 128), seed=79, scale=0.5)
+    cache.append(slots, to_bf16(k16, dev), to_bf16(v16, dev))
+    for b, s in enumerate(slots_l):
+        if s >= 0: hist[s] = (np.concatenate([hist[s][0], k16[b:b + 1]]), np.concatenate([hist[s][1], v16[b:b + 1]]))
+    out = O.bf16_to_f32(to_u16(cache.attention(to_bf16(q16, dev), slots, SCALE, nsplit=3)))
+    for b in (0, 7, 33, 71):
+        s = slots_l[b]
+        ref = O.ref_attention(q16[b], hist[s][0], hist[s][1], SCALE)
+        assert np.abs(out[b] - ref).max() <= 2e-2 * np.abs(ref).max() + 1e-3
+        dk, dv = cache.decompress(s)
+        assert np.array_equal(to_u16(dk), hist[s][0]) and np.array_equal(to_u16(dv), hist[s][1])
+    cache.check_capacity()
