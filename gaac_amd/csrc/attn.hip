@@ -370,7 +370,7 @@ __device__ __forceinline__ void load_tags(const Bases& B, const TileTable& TT, i
     Tg.vfl = reinterpret_cast<const u32*>(B.vov + (size_t)Tg.vto * (size_t)B.TS + SLOT_FL)[a];
   } else {
     const unsigned w = (unsigned)(tile * T + a);
-    Tg.kfl = (u32)B.kfl[w]; Tg.vfl = (u32)B.vfl[w];
+    Tg.kfl = (u32)__builtin_nontemporal_load(B.kfl + w); Tg.vfl = (u32)__builtin_nontemporal_load(B.vfl + w);
     Tg.kto = (u32)B.kto[tile]; Tg.vto = (u32)B.vto[tile];
     Tg.raw = 0;
   }
@@ -640,19 +640,22 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
   // split it would finish long before the other, which then runs alone and cannot hide its own latencies.  Ping-pong registers
   // R0/R1; tag words are fetched one tile further ahead; indices past the end are clamped for the loads (no load sits under a
   // branch the consumer has to join) and not consumed.  A partly filled last tile of the sequence is handled at the end by wave 0.
+  // logical tile index i of this block -> tile tlo + i
+  const int full = ntiles - ((S % T) != 0 ? 1 : 0);      // tiles with all 16 rows
+  const int n_own = max(min(thi, full) - tlo, 0);
   const bool part_here = (S % T) != 0 && thi == ntiles && thi > tlo;
-  const int thd = thi - (part_here ? 1 : 0);
-  const int tcl = max(thd - 1, tlo);
-  int tA = tlo + wave, tB = tA + NW;
+  const int icl = max(n_own - 1, 0);
+#define TILE(i) (tlo + (i))
+  int iA = wave, iB = wave + NW;
   TileRegs R0, R1;
   TagRegs Tg, TgC0, TgC1;
-  if (tA < thd) {          // start the first tile's loads before waiting for the block tables
-    load_tags<PAGED>(B, TT, tA, a, Tg);
+  if (iA < n_own) {          // start the first tile's loads before waiting for the block tables
+    load_tags<PAGED>(B, TT, TILE(iA), a, Tg);
     TgC0 = Tg;
-    load_tile<PAGED>(B, tA, lane, Tg, R0);
-    load_tags<PAGED>(B, TT, min(tB, tcl), a, Tg);
+    load_tile<PAGED>(B, TILE(iA), lane, Tg, R0);
+    load_tags<PAGED>(B, TT, TILE(min(iB, icl)), a, Tg);
   }
-  if (tid == 0) next_tile = tlo + 2 * NW;
+  if (tid == 0) next_tile = 2 * NW;
   GAAC_STAMP(6);
   if (tid < 256) tables_store(L, Tr, tid, G);
   GAAC_STAMP(7);
@@ -681,26 +684,27 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
     }
   }
 
-  if (tA < thd) {
-    int vC = take_tile(&next_tile, thd, lane);
-    while (true) {        // R0 = tile tA, Tg = tags of tile tB
+  if (iA < n_own) {
+    int vC = take_tile(&next_tile, n_own, lane);
+    while (true) {        // R0 = tile iA, Tg = tags of tile iB
       TgC1 = Tg;
-      load_tile<PAGED>(B, min(tB, tcl), lane, Tg, R1);
-      const int vD = take_tile(&next_tile, thd, lane);
-      const int tC = uniform_tile(vC);
-      load_tags<PAGED>(B, TT, min(tC, tcl), a, Tg);
-      if (!PAGED || !TgC0.raw) consume<PAGED, false>(R0, st, L, B, TgC0.kto, TgC0.vto, tA, S, A.scale_log2e, a, q, qf);
-      if (tB >= thd) break;
+      load_tile<PAGED>(B, TILE(min(iB, icl)), lane, Tg, R1);
+      const int vD = take_tile(&next_tile, n_own, lane);
+      const int iC = uniform_tile(vC);
+      load_tags<PAGED>(B, TT, TILE(min(iC, icl)), a, Tg);
+      if (!PAGED || !TgC0.raw) consume<PAGED, false>(R0, st, L, B, TgC0.kto, TgC0.vto, TILE(iA), S, A.scale_log2e, a, q, qf);
+      if (iB >= n_own) break;
       TgC0 = Tg;
-      load_tile<PAGED>(B, min(tC, tcl), lane, Tg, R0);
-      const int vE = take_tile(&next_tile, thd, lane);
-      const int tD = uniform_tile(vD);
-      load_tags<PAGED>(B, TT, min(tD, tcl), a, Tg);
-      if (!PAGED || !TgC1.raw) consume<PAGED, false>(R1, st, L, B, TgC1.kto, TgC1.vto, tB, S, A.scale_log2e, a, q, qf);
-      if (tC >= thd) break;
-      tA = tC; tB = tD; vC = vE;
+      load_tile<PAGED>(B, TILE(min(iC, icl)), lane, Tg, R0);
+      const int vE = take_tile(&next_tile, n_own, lane);
+      const int iD = uniform_tile(vD);
+      load_tags<PAGED>(B, TT, TILE(min(iD, icl)), a, Tg);
+      if (!PAGED || !TgC1.raw) consume<PAGED, false>(R1, st, L, B, TgC1.kto, TgC1.vto, TILE(iB), S, A.scale_log2e, a, q, qf);
+      if (iC >= n_own) break;
+      iA = iC; iB = iD; vC = vE;
     }
   }
+#undef TILE
   GAAC_STAMP(2);
 #ifdef GAAC_PHASE_TIMING
   if (A.dbg && lane == 0) A.dbg[((long)gridDim.x + blockIdx.x) * 8 + wave] = wall_clock64();
@@ -830,9 +834,9 @@ struct RawTile { u32x4 k[4], v[4]; };
 __device__ __forceinline__ void load_raw_tile(const u16* __restrict__ kh, const u16* __restrict__ vh, int tile, int S, int a, int q, RawTile& R) {
   const int kt = min(tile * T + a, S - 1);
 #pragma unroll
-  for (int j = 0; j < 4; ++j) R.k[j] = *reinterpret_cast<const u32x4*>(kh + (long)kt * D + 32 * j + 8 * q);
+  for (int j = 0; j < 4; ++j) R.k[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(kh + (long)kt * D + 32 * j + 8 * q));
 #pragma unroll
-  for (int r = 0; r < 4; ++r) R.v[r] = *reinterpret_cast<const u32x4*>(vh + (long)min(tile * T + 4 * q + r, S - 1) * D + 8 * a);
+  for (int r = 0; r < 4; ++r) R.v[r] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(vh + (long)min(tile * T + 4 * q + r, S - 1) * D + 8 * a));
 }
 template <bool PARTIAL>
 __device__ __forceinline__ void consume_raw_tile(const RawTile& R, WaveState& st, int tile, int S, float scale_log2e, int q, const u32x4 (&qf)[4]) {
