@@ -23,7 +23,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the attention kernel on the default workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by the
 # library's plain 64 MiB copy kernel (factors 1.99937 read, 1.0 write); the profiler runs are separate from a timing run, so the
 # figure is carried here and reported only for the configuration it was measured on.
-MEASURED_TRAFFIC = {"nsplit": 32, "copies": 3, "bytes": 193073971}
+MEASURED_TRAFFIC = {"nsplit": 32, "copies": 3, "bytes": 194721485}
 
 
 def make_kv(seed: int, H: int, S: int, lo: float = -4.0, hi: float = 4.0) -> torch.Tensor:
