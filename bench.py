@@ -23,7 +23,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the attention kernel on the default workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by the
 # library's plain 64 MiB copy kernel (factors 1.99937 read, 1.0 write); the profiler runs are separate from a timing run, so the
 # figure is carried here and reported only for the configuration it was measured on.
-MEASURED_TRAFFIC = {"nsplit": 32, "copies": 3, "bytes": 194721485}
+MEASURED_TRAFFIC = {"nsplit": 32, "bytes": 194669694}
 
 
 def make_kv(seed: int, H: int, S: int, lo: float = -4.0, hi: float = 4.0) -> torch.Tensor:
@@ -77,7 +77,7 @@ def cpu_baseline(k16: np.ndarray, v16: np.ndarray, q16: np.ndarray, b3k, b4k, b3
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1); ap.add_argument("--steps", type=int, default=300); ap.add_argument("--warmup", type=int, default=30)
-    ap.add_argument("--copies", type=int, default=3); ap.add_argument("--nsplit", type=int, default=0)
+    ap.add_argument("--copies", type=int, default=6); ap.add_argument("--nsplit", type=int, default=0)
     ap.add_argument("--batch", type=int, default=1, help="decode64k only: batch rows (each with its own 65536-token context); the headline is 1")
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="also run the library's plain 64 MiB copy kernel 10 times (the known-size kernel for scaling FETCH_SIZE / WRITE_SIZE)")
@@ -263,13 +263,14 @@ def bench_codec(a):
     b3, b4 = O.calibrate(x16[:, :1024], 8); op = O.encode(x16, "k", b3, b4, 8); t1 = time.perf_counter(); od = O.decode(op); t2 = time.perf_counter()
     same = np.array_equal(od, x16) and int(op.ovf_head_start[-1]) == int(page.ovf_head_start[-1]) and np.array_equal(b3, codec.base3.cpu().numpy())
     # the encoder and decoder kernels alone at the page size of config 1 (K and V [8, 65536, 128]), events around each launch, the
-    # inputs rotating over 3 copies; bytes = BF16 rows on one side + Page.nbytes on the other
+    # inputs rotating over --copies copies; bytes = BF16 rows on one side + Page.nbytes on the other
     from gaac_amd.codec import CB as _CB, row_offsets
     full = {}
     for kind, seed in (("k", 1), ("v", 2)):
-        x0 = make_kv(seed, N_KV, S_CTX).to(dev); xs = [x0, x0.clone(), x0.clone()]
+        nc = a.copies
+        x0 = make_kv(seed, N_KV, S_CTX).to(dev); xs = [x0] + [x0.clone() for _ in range(nc - 1)]
         c1 = Codec(N_KV).calibrate(x0[:, :1024]); e1 = TileEncoder(kind)
-        pgs = [e1.encode(c1, x0)]; pgs += [clone_store(pgs[0]), clone_store(pgs[0])]
+        pgs = [e1.encode(c1, x0)]; pgs += [clone_store(pgs[0]) for _ in range(nc - 1)]
         smb = torch.empty(N_KV, S_CTX * D, dtype=torch.uint8, device=dev); cdb = torch.empty(N_KV, S_CTX * _CB, dtype=torch.uint8, device=dev)
         flb = torch.zeros(N_KV, S_CTX, dtype=torch.int32, device=dev)
         nb = x0.numel() * 2 + pgs[0].nbytes
@@ -280,12 +281,12 @@ def bench_codec(a):
                 e0.record(); fn(i); e1_.record()
             torch.cuda.synchronize()
             return float(np.median([e0.elapsed_time(e1_) * 1e3 for e0, e1_ in es]))
-        te = ev(lambda i: e1.encode_tiles(xs[i % 3], c1.base3, c1.base4, smb, cdb, flb, S_CTX, S_CTX, N_KV))
+        te = ev(lambda i: e1.encode_tiles(xs[i % nc], c1.base3, c1.base4, smb, cdb, flb, S_CTX, S_CTX, N_KV))
         tb = e1.encode_tiles(x0, c1.base3, c1.base4, smb, cdb, flb, S_CTX, S_CTX, N_KV)
         ovf = torch.zeros_like(pgs[0].ovf)
         tc = ev(lambda i: e1.compact(tb, pgs[0].ovf_head_start, ovf))
-        td = ev(lambda i: Codec.decode(pgs[i % 3]))
-        tr = ev(lambda i: row_offsets(pgs[i % 3].flags, S_CTX))
+        td = ev(lambda i: Codec.decode(pgs[i % nc]))
+        tr = ev(lambda i: row_offsets(pgs[i % nc].flags, S_CTX))
         full[kind] = {"encode_tiles_us": round(te, 1), "encode_GBps": round(nb / te / 1e3, 1), "encode_frac_of_hbm_peak": round(nb / te / 1e3 / HBM_PEAK_GBS, 3),
                       "compact_us": round(tc, 1), "decode_us": round(td, 1), "decode_GBps": round(nb / td / 1e3, 1),
                       "decode_frac_of_hbm_peak": round(nb / td / 1e3 / HBM_PEAK_GBS, 3), "row_offsets_us": round(tr, 1), "bytes_in_plus_out": nb}
