@@ -369,9 +369,9 @@ __device__ __forceinline__ void load_tags(const Bases& B, const TileTable& TT, i
     Tg.kfl = reinterpret_cast<const u32*>(B.kov + (size_t)Tg.kto * (size_t)B.TS + SLOT_FL)[a];
     Tg.vfl = reinterpret_cast<const u32*>(B.vov + (size_t)Tg.vto * (size_t)B.TS + SLOT_FL)[a];
   } else {
-    const unsigned w = (unsigned)(tile * T + a);
+    const u32 w = (u32)(tile * T + a);
     Tg.kfl = (u32)__builtin_nontemporal_load(B.kfl + w); Tg.vfl = (u32)__builtin_nontemporal_load(B.vfl + w);
-    Tg.kto = (u32)B.kto[tile]; Tg.vto = (u32)B.vto[tile];
+    Tg.kto = (u32)B.kto[(u32)tile]; Tg.vto = (u32)B.vto[(u32)tile];
     Tg.raw = 0;
   }
 }
@@ -385,8 +385,18 @@ __device__ __forceinline__ void load_tile(const Bases& B, int tile, int lane, co
     load_payload(ks, ks + SLOT_CD, lane, R.k.pay);
     load_payload(vs, vs + SLOT_CD, lane, R.v.pay);
   } else {
-    load_payload(B.ksm + (size_t)tile * TILE_SM, B.kcd + (size_t)tile * TILE_CD, lane, R.k.pay);
-    load_payload(B.vsm + (size_t)tile * TILE_SM, B.vcd + (size_t)tile * TILE_CD, lane, R.v.pay);
+    // uniform 64-bit base + 32-bit byte offset per lane (one add per array; a head's arrays stay below 4 GiB, checked on the host)
+    const u32 so = (u32)tile * TILE_SM + 16u * (u32)lane, co = (u32)tile * TILE_CD + 4u * (u32)lane;
+    R.k.pay.s0 = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(B.ksm + so));
+    R.k.pay.s1 = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(B.ksm + so + 1024u));
+    R.v.pay.s0 = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(B.vsm + so));
+    R.v.pay.s1 = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(B.vsm + so + 1024u));
+    R.k.pay.c0 = __builtin_nontemporal_load(reinterpret_cast<const u32*>(B.kcd + co));
+    R.k.pay.c1 = __builtin_nontemporal_load(reinterpret_cast<const u32*>(B.kcd + co + 256u));
+    R.k.pay.c2 = __builtin_nontemporal_load(reinterpret_cast<const u32*>(B.kcd + co + 512u));
+    R.v.pay.c0 = __builtin_nontemporal_load(reinterpret_cast<const u32*>(B.vcd + co));
+    R.v.pay.c1 = __builtin_nontemporal_load(reinterpret_cast<const u32*>(B.vcd + co + 256u));
+    R.v.pay.c2 = __builtin_nontemporal_load(reinterpret_cast<const u32*>(B.vcd + co + 512u));
   }
   // escape bytes per line of K (low half) and V (high half): one scan for both
   const u32 rb = (u32)esc_bytes(Tg.kfl) | ((u32)esc_bytes(Tg.vfl) << 16);
@@ -394,8 +404,13 @@ __device__ __forceinline__ void load_tile(const Bases& B, int tile, int lane, co
   R.k.f = Tg.kfl; R.v.f = Tg.vfl;
   R.k.pos0 = (excl & 0xFFFFu) + (u32)esc_prefix(Tg.kfl, 8 * q);
   R.v.pos0 = (excl >> 16) + (u32)esc_prefix(Tg.vfl, 8 * q);
-  R.k.e = load_u32x2_unaligned(esc_of_tile<PAGED>(B.kov, PAGED ? __builtin_amdgcn_readfirstlane(Tg.kto) : Tg.kto, B.TS) + R.k.pos0);
-  R.v.e = load_u32x2_unaligned(esc_of_tile<PAGED>(B.vov, PAGED ? __builtin_amdgcn_readfirstlane(Tg.vto) : Tg.vto, B.TS) + R.v.pos0);
+  if (PAGED) {
+    R.k.e = load_u32x2_unaligned(esc_of_tile<PAGED>(B.kov, __builtin_amdgcn_readfirstlane(Tg.kto), B.TS) + R.k.pos0);
+    R.v.e = load_u32x2_unaligned(esc_of_tile<PAGED>(B.vov, __builtin_amdgcn_readfirstlane(Tg.vto), B.TS) + R.v.pos0);
+  } else {      // stream base (uniform) + 32-bit offset (tile offset + position in the tile)
+    R.k.e = load_u32x2_unaligned(B.kov + (u32)(Tg.kto + R.k.pos0));
+    R.v.e = load_u32x2_unaligned(B.vov + (u32)(Tg.vto + R.v.pos0));
+  }
 }
 
 // ---------------------------------------------------------------------------------------------------- one tile pair
@@ -975,6 +990,7 @@ static int attn_split_impl(
   GAAC_REQUIRE(!has_tail || (vt && TL && TCAP >= 1 && TCAP <= T), "gaac_attn: tail needs kt, vt, TL and 1 <= TCAP <= %d", T);
   const int nslot = nsplit;
   GAAC_REQUIRE(nsplit >= 1 && nslot <= MAX_SLOTS, "gaac_attn: nsplit must be in 1..%d", MAX_SLOTS);
+  GAAC_REQUIRE(S_pad > 0 && S_pad <= (1 << 24), "gaac_attn: at most %d tokens per cache head (32-bit byte offsets inside a head)", 1 << 24);
   AttnArgs A;
   A.k = StoreView{smk, ck, fk, tok, ovk, ohsk, b3k, b4k};
   A.v = StoreView{smv, cv, fv, tov, ovv, ohsv, b3v, b4v};
