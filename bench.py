@@ -23,7 +23,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the attention kernel on the default workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by the
 # library's plain 64 MiB copy kernel (factors 1.99937 read, 1.0 write); the profiler runs are separate from a timing run, so the
 # figure is carried here and reported only for the configuration it was measured on.
-MEASURED_TRAFFIC = {"nsplit": 32, "bytes": 194669694}
+MEASURED_TRAFFIC = {"nsplit": 32, "bytes": 194632199}
 
 
 def make_kv(seed: int, H: int, S: int, lo: float = -4.0, hi: float = 4.0) -> torch.Tensor:
@@ -76,7 +76,7 @@ def cpu_baseline(k16: np.ndarray, v16: np.ndarray, q16: np.ndarray, b3k, b4k, b3
 
 def main():
     ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1); ap.add_argument("--steps", type=int, default=300); ap.add_argument("--warmup", type=int, default=30)
+    ap.add_argument("--gpus", type=int, default=1); ap.add_argument("--steps", type=int, default=1000); ap.add_argument("--warmup", type=int, default=30)
     ap.add_argument("--copies", type=int, default=6); ap.add_argument("--nsplit", type=int, default=0)
     ap.add_argument("--batch", type=int, default=1, help="decode64k only: batch rows (each with its own 65536-token context); the headline is 1")
     ap.add_argument("--traffic-calibration", action="store_true",
@@ -110,7 +110,8 @@ def main():
     k_all, v_all = make_kv(1, H, S_CTX + TAIL_TOK), make_kv(2, H, S_CTX + TAIL_TOK, *v_range)
     q = torch.randn(B, n_q, D, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
     kd, vd, qd = k_all.to(dev), v_all.to(dev), q.to(dev)
-    ck, cv = Codec(N_KV).calibrate(kd[:, :1024]), Codec(N_KV).calibrate(vd[:, :1024])
+    # bases per cache head (for one batch row that is per kv head; more rows are separate sequences with their own calibration, as in the cache)
+    ck, cv = Codec(H).calibrate(kd[:, :1024]), Codec(H).calibrate(vd[:, :1024])
     kp = TileEncoder("k").encode(ck, kd[:, :S_CTX].contiguous()); vp = TileEncoder("v").encode(cv, vd[:, :S_CTX].contiguous())
     kt = torch.zeros(H, 16, D, dtype=torch.bfloat16, device=dev); vt = torch.zeros_like(kt)
     kt[:, :TAIL_TOK] = kd[:, S_CTX:]; vt[:, :TAIL_TOK] = vd[:, S_CTX:]
@@ -122,7 +123,7 @@ def main():
     q2d = qd.reshape(B * n_q, D).contiguous()
     S_pad = kp.sm.shape[1] // D
     pages = [(kp, vp)] + [(clone_store(kp), clone_store(vp)) for _ in range(a.copies - 1)]
-    alg_bytes = kp.nbytes + vp.nbytes + 2 * H * TAIL_TOK * D * 2 + 2 * B * n_q * D * 2 + 4 * N_KV * D
+    alg_bytes = kp.nbytes + vp.nbytes + 2 * H * TAIL_TOK * D * 2 + 2 * B * n_q * D * 2 + 4 * H * D
     bf16_bytes = 2 * H * (S_CTX + TAIL_TOK) * D * 2 + 2 * B * n_q * D * 2
 
     def step(i, phase="fused"):
@@ -167,7 +168,7 @@ def main():
     # ---- duration of the attention kernel itself: HIP events on the launch stream around batches of back-to-back launches
     # (one event pair per launch would add the event's own ~3 us to every sample)
     BATCH = 20
-    nb = max(5, a.steps // BATCH)
+    nb = min(max(5, a.steps // BATCH), 30)
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nb)]
     for b_, (e0, e1) in enumerate(evs):
         e0.record()
@@ -184,17 +185,22 @@ def main():
     kb = [kd.clone() for _ in range(a.copies)]; vb = [vd.clone() for _ in range(a.copies)]
     qb = qd.view(B, n_q, D)
     ref_b = bf16_attention(qb, kb[0], vb[0], scale).float().view(B * n_q, D)
-    assert (ref_b - ref).abs().max().item() <= 1e-2, "baseline kernel is off"
+    assert (ref_b - ref).abs().max().item() <= 2e-2 * ref.abs().max().item() + 1e-3, "baseline kernel is off"      # the reference's tolerance
     bf16_us, bf16_ns = None, None
     for ns in sorted({max(1, x // B) for x in (64, 96, 128, 192)}):
         wsb = AttnWorkspace(B * n_q, ns, torch.bfloat16, dev)
-        for i in range(10): bf16_attention(qb, kb[i % a.copies], vb[i % a.copies], scale, ns, wsb)
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        n_b = max(60, a.steps // 2)
-        e0.record()
-        for i in range(n_b): bf16_attention(qb, kb[i % a.copies], vb[i % a.copies], scale, ns, wsb)
-        e1.record(); torch.cuda.synchronize()
-        t = e0.elapsed_time(e1) * 1e3 / n_b
+        outb = torch.empty(B * n_q, D, dtype=torch.bfloat16, device=dev)
+        for i in range(10): bf16_attention(qb, kb[i % a.copies], vb[i % a.copies], scale, ns, wsb, out=outb)
+        n_b = min(max(60, a.steps // 2), 300)
+        gb = torch.cuda.CUDAGraph()                      # timed like the compressed kernel: one graph of launches, wall clock
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            with torch.cuda.graph(gb, stream=side):
+                for i in range(n_b): bf16_attention(qb, kb[i % a.copies], vb[i % a.copies], scale, ns, wsb, out=outb)
+        torch.cuda.synchronize(); gb.replay(); torch.cuda.synchronize()
+        t0b = time.perf_counter(); gb.replay(); torch.cuda.synchronize()
+        t = (time.perf_counter() - t0b) * 1e6 / n_b
+        del gb
         if bf16_us is None or t < bf16_us: bf16_us, bf16_ns = t, ns
     q4 = qd.view(B, n_q, 1, D)
     k4 = [x.view(B, N_KV, S_CTX + TAIL_TOK, D) for x in kb]; v4 = [x.view(B, N_KV, S_CTX + TAIL_TOK, D) for x in vb]
