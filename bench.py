@@ -128,7 +128,7 @@ def main():
 
     def step(i, phase="fused"):
         K, V = pages[i % len(pages)]
-        return attn_launch(K, V, q2d, slots, n_q, N_KV, SL, S_pad, scale, nsplit, kt, vt, TL, 16, ws=ws, phase=phase)
+        return attn_launch(K, V, q2d, None, n_q, N_KV, SL, S_pad, scale, nsplit, kt, vt, TL, 16, ws=ws, phase=phase)      # rows in order, as gaac.kernel.attention
 
     if a.traffic_calibration:
         from gaac_amd import _lib

@@ -617,7 +617,8 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
   // Level 1: the slot of the batch row; the query rows do not depend on it
   TableRegs Tr;
   if (tid < 256) tables_load_q(Tr, tid, A.q + qh0 * D, G);
-  const int slot = PAGED ? 0 : A.slot[b], ch = PAGED ? kvh : (slot < 0 ? 0 : slot) * A.n_kv + kvh;
+  // (no slot map = row b attends over cache heads b*n_kv ..: one level of dependent loads less)
+  const int slot = PAGED ? 0 : (A.slot ? A.slot[b] : b), ch = PAGED ? kvh : (slot < 0 ? 0 : slot) * A.n_kv + kvh;
   // Level 2: everything indexed by the cache head
   int S, TLh = 0; long khs = 0, vhs = 0;
   if (PAGED) S = S_ranked >= 0 ? S_ranked : max(A.sl[b], 0);
@@ -984,7 +985,7 @@ static int attn_split_impl(
     const void* kt, const void* vt, const int* TL, int TCAP, float* pm, float* pl, float* pa, int* tickets, void* out, void* stream) {
   GAAC_REQUIRE(n_kv > 0 && n_q > 0 && n_q % n_kv == 0 && n_q / n_kv >= 1 && n_q / n_kv <= GMAX, "GQA group size must be 1..%d (n_q=%d, n_kv=%d)", GMAX, n_q, n_kv);
   GAAC_REQUIRE(smk && ck && fk && tok && ovk && ohsk && b3k && b4k && smv && cv && fv && tov && ovv && ohsv && b3v && b4v, "gaac_attn: null store pointer");
-  GAAC_REQUIRE(q && slot && SL && pm && pl && pa, "gaac_attn: null pointer");
+  GAAC_REQUIRE(q && SL && pm && pl && pa, "gaac_attn: null pointer");
   GAAC_REQUIRE(B > 0 && S_pad > 0 && S_pad % T == 0 && NB > 0, "gaac_attn: bad sizes B=%d S_pad=%d NB=%d", B, S_pad, NB);
   const bool has_tail = kt != nullptr;
   GAAC_REQUIRE(!has_tail || (vt && TL && TCAP >= 1 && TCAP <= T), "gaac_attn: tail needs kt, vt, TL and 1 <= TCAP <= %d", T);

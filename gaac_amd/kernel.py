@@ -52,7 +52,7 @@ def attn_launch(K, V, q2d, slots, n_q, n_kv, SL, S_pad, scale, nsplit, kt=None, 
         raise RuntimeError(f"GQA group size must be 1..{GMAX}")
     if q2d.shape[-1] != D:
         raise RuntimeError("head_dim must be 128")
-    B = slots.shape[0]
+    B = slots.shape[0] if slots is not None else q2d.shape[0] // n_q      # slots=None: row b attends over cache heads b*n_kv ..
     has_tail = kt is not None and kt.numel() > 0
     nslot = nsplit        # the raw tail is folded into the last split's partial
     if ws is None:
@@ -83,9 +83,8 @@ def attention(q, kp, vp, scale=None, nsplit=None, phase="fused"):
     n_kv = kp.H // B
     dev = q.device
     if nsplit is None: nsplit = choose_nsplit(B, n_kv, kp.S)
-    slots = torch.arange(B, dtype=torch.int32, device=dev)
     SL = torch.full((kp.H,), kp.S, dtype=torch.int32, device=dev)
-    out = attn_launch(kp, vp, q.reshape(B * n_q, Dq).contiguous(), slots, n_q, n_kv, SL, kp.sm.shape[1] // D,
+    out = attn_launch(kp, vp, q.reshape(B * n_q, Dq).contiguous(), None, n_q, n_kv, SL, kp.sm.shape[1] // D,
                       scale if scale is not None else Dq ** -0.5, nsplit, phase=phase)
     return out.view(B, n_q, Dq)
 

@@ -53,7 +53,7 @@ int gaac_decode_tiles(int kind, const uint8_t* sm, const uint8_t* codes, const i
                       int S_pad, void* out, long out_head_stride, long out_row_stride, void* stream);
 
 /* gaac_attn_launch, /root/reference/gaac/kernel.py:296-326 (kernels :48-294).  Same 16 store tensors, q [B*n_q, 128] bf16,
- * slot map [B] (slot < 0 = padded row, output 0), SL [cache heads] compressed tokens per head, S_pad = token stride of a
+ * slot map [B] (slot < 0 = padded row, output 0; NULL = the identity, row b attends over cache heads b*n_kv ..), SL [cache heads] compressed tokens per head, S_pad = token stride of a
  * head, nsplit, and the optional raw tail kt/vt [cache heads, TCAP, 128] bf16 with lengths TL (kt == NULL: no tail).
  * NB = rows of the base tables (n_kv, or the number of cache heads for per-sequence bases).
  * Differences from the reference entry: the caller passes the partial buffers pm, pl [B*n_q*NSLOT] and
