@@ -34,7 +34,8 @@ struct AttnArgs {
   const int* slot; const int* sl;
   int S_pad; float scale_log2e; int nsplit; int nslot; int n_kv; int n_q; int G; int NB;
   const u16* kt; const u16* vt; const int* tl; int tcap;
-  int* tickets; u16* out;      // fused merge: one arrival counter per (batch row, kv head), zero between launches
+  u32* epochs; u16* out;       // fused merge: the word with the epoch of the last merged launch; pm / pl / pa then hold 64-bit records
+  int S_all;                   // >= 0: every addressed cache head holds exactly S_all compressed tokens (sl is not read)
   // paged slot pool (k_attn_split<true>): sl = tokens per batch row, bt = block table [B][bt_stride], mt = mode table, pool = tile
   // slots of TS bytes, raw = side pool of BF16 tiles; physical tile = block*2*n_kv + 2*kvh + kind
   const uint8_t* pool; const u16* raw; const int* mt; const int* bt; int bt_stride; int TS;
@@ -44,8 +45,10 @@ struct AttnArgs {
 };
 #ifdef GAAC_PHASE_TIMING
 #define GAAC_STAMP(k) do { if (A.dbg && threadIdx.x == 0) A.dbg[(long)blockIdx.x * 8 + (k)] = wall_clock64(); } while (0)
+#define GAAC_MSTAMP(k, v) do { if (A.dbg && threadIdx.x == 0) A.dbg[(2 * (long)gridDim.x + blockIdx.x) * 8 + (k)] = (v); } while (0)
 #else
 #define GAAC_STAMP(k) do {} while (0)
+#define GAAC_MSTAMP(k, v) do {} while (0)
 #endif
 constexpr int MAX_CHUNK = 1024;  // tiles per split whose slot lookups a block keeps in LDS (paged mode)
 constexpr int SLOT_CD = TILE_SM, SLOT_FL = TILE_SM + TILE_CD, SLOT_OV = SLOT_FL + 4 * T;      // byte offsets inside a tile slot
@@ -58,89 +61,129 @@ __device__ __forceinline__ u32 pack_bf16x2(float lo, float hi) {
 }
 
 // ---------------------------------------------------------------------------------------------------- fused merge
-// Merge of the split partials (gaac_combine, /root/reference/gaac/kernel.py:281-294) by the LAST block of a (batch row, kv head)
-// to finish: every block publishes its partial, then takes a ticket; the block that draws the last ticket merges all NSLOT
-// partials of the G query heads and re-arms the counter.  One wave per head, no block-wide synchronisation inside.
-// The partials travel between blocks on different XCDs (one L2 each) inside one kernel, so they are written and read with
-// agent-scope accesses (write-through stores, cache-bypassing loads) instead of whole-L2 write-back/invalidate fences.
+// Merge of the split partials (gaac_combine, /root/reference/gaac/kernel.py:281-294) inside the split kernel, by ONE block of each
+// (batch row, kv head), without atomics and without any block waiting for a store acknowledgement on its way out:
+//
+//   * One word, *epoch, holds the epoch of the last merged launch.  Every block reads it while its first tiles are in flight; this
+//     launch's EPOCH is that value + 1, the same for all blocks (only the last block of the grid writes the word, as its very last
+//     action; it is the last to start, so every block has read the word long before).  Records of any earlier launch, whatever its
+//     shape, carry a smaller epoch.
+//   * A partial value travels as one 64-bit record (fp32 bits | epoch << 32) written with a single 64-bit store: a reader sees either
+//     the whole record of this launch or an older one, never a torn one (naturally aligned 64-bit accesses are single-copy atomic),
+//     so no fence, flag or acknowledgement orders data against a separate signal.  Records are written with agent-scope stores
+//     (write-through) and read with agent-scope loads (they bypass the reader's L2): the blocks of a head sit on different XCDs.
+//   * The MERGERS are the head's last (up to eight) blocks in index order; each takes a share of the head's output (half a query head
+//     per wave), because one CU pulls records at only ~80 GB/s.  Once a merger has stored its own partial it loads the records of its
+//     share from all blocks of the head and re-reads those whose epoch is not yet the launch's.  Workgroups start in index order and
+//     a head's blocks are consecutive, so everything a merger waits for is running, done, or one of the at most seven later mergers
+//     of the same head, which get the next free CUs; blocks that are not mergers wait for nobody.  The wait is bounded all the same
+//     (MERGE_SPIN_LIMIT re-reads, then the rows are written as NaN), so that neither a damaged epoch word nor another start order
+//     can hang the GPU.
+//   * Launches that share the records and the epoch word must be ordered on one stream.  To re-arm after a failed launch, zero both.
 typedef __attribute__((ext_vector_type(4))) float f32x4v;
 __device__ __forceinline__ void store_partial(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
-constexpr int AUX_AGENT_SCOPE = 0x10;      // sc1 of the gfx94x/gfx950 buffer cache policy
-__device__ __forceinline__ void merge_head_by_wave(const AttnArgs& A, long row, float* __restrict__ fs, int lane) {
-  // The m/l loads and the first 32 partial rows are issued before the first result is needed (one memory round trip for them).
-  // Buffer loads past the end of a row's partials return zero without a branch.
-  const int nslot = A.nslot;
-  const __amdgpu_buffer_rsrc_t rm = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(A.pm + row * nslot), 0, nslot * 4, 0x00027000);
-  const __amdgpu_buffer_rsrc_t rl = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(A.pl + row * nslot), 0, nslot * 4, 0x00027000);
-  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(A.pa + row * nslot * D), 0, nslot * D * 4, 0x00027000);
-  constexpr int PER = MAX_SLOTS / 64, CH = 16;
-  const int sg = lane >> 5, dq = (lane & 31) * 4;      // two slots per wave-wide load, four dims per lane
-  u32 mv[PER], lv[PER];
+__device__ __forceinline__ void ll_store(u64* p, float v, u32 epoch) {
+  __hip_atomic_store(p, (u64)__float_as_uint(v) | ((u64)epoch << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ u64 ll_load(const u64* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ bool ll_stale(u64 r, u32 epoch) { return (u32)(r >> 32) != epoch; }
+__device__ __forceinline__ float ll_value(u64 r) { return __uint_as_float((u32)r); }
+constexpr int MERGE_SPIN_LIMIT = 1 << 16;      // re-reads of a chunk before the merger gives up (each with a short sleep: ~0.1 s)
+// (no branch around the load: a load under a branch is waited for where the branch ends, together with everything issued before it)
+__device__ __forceinline__ u32 load_epoch(const AttnArgs& A, int bh) {
+  const u32* p = A.epochs ? A.epochs : reinterpret_cast<const u32*>(A.q);
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+}
+// A block barrier that orders LDS traffic only.  (__syncthreads() also waits for the block's global stores to be acknowledged,
+// which for write-through stores is a trip to memory.)
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// LDS of a merging block: per wave the (m, then factor) and l of every slot; the waves' partial sums and their verdicts.
+template <int NW> struct MergeScratch { float f[NW][MAX_SLOTS], l[NW][MAX_SLOTS]; float part[NW][64]; int ok[NW]; };
+
+// One merger's work for half a query head (64 output dims, one per lane), shared by the NW waves of the block: every wave reads the
+// m / l records of all slots (lane = slot) and the accumulator records of slots wave, wave + NW, ...; the waves' sums meet in LDS.
+// The code is kept short on purpose: it runs once per launch on a cold instruction cache, where straight-line code costs a trip to
+// the L2 per cache line.  Called by all threads of the block.
+template <int NW>
+__device__ __forceinline__ void merge_half_head(const AttnArgs& A, long row, int half, u32 epoch, MergeScratch<NW>& X, int wave, int lane) {
+  const int nslot = A.nslot, d = 64 * half + lane;
+  const u64* rm = reinterpret_cast<const u64*>(A.pm) + row * nslot;
+  const u64* rl = reinterpret_cast<const u64*>(A.pl) + row * nslot;
+  const u64* ra = reinterpret_cast<const u64*>(A.pa) + row * nslot * D + d;
+  float* fs = X.f[wave]; float* ls = X.l[wave];
+  constexpr int CH = 4;
+  bool ok = true;
+  // all loads of the first round are issued before the first use: the wave's first CH accumulator rows, then m / l of slots 0..63
+  u64 v[CH];
 #pragma unroll
-  for (int k = 0; k < PER; ++k) {
-    mv[k] = __builtin_amdgcn_raw_buffer_load_b32(rm, (lane + 64 * k) * 4, 0, AUX_AGENT_SCOPE);
-    lv[k] = __builtin_amdgcn_raw_buffer_load_b32(rl, (lane + 64 * k) * 4, 0, AUX_AGENT_SCOPE);
-  }
-  u32x4 v[CH];
-#pragma unroll
-  for (int k = 0; k < CH; ++k) v[k] = __builtin_amdgcn_raw_buffer_load_b128(ra, ((sg + 2 * k) * D + dq) * 4, 0, AUX_AGENT_SCOPE);
+  for (int k = 0; k < CH; ++k) { const int s = wave + NW * k; v[k] = s < nslot ? ll_load(ra + (long)s * D) : 0ull; }
   float m = -INFINITY;
-#pragma unroll
-  for (int k = 0; k < PER; ++k) m = fmaxf(m, lane + 64 * k < nslot ? __uint_as_float(mv[k]) : -INFINITY);
+  for (int s0 = 0; s0 < nslot; s0 += 64) {      // one pass for up to 64 splits
+    const int s = s0 + lane;
+    u64 mr = s < nslot ? ll_load(rm + s) : 0ull, lr = s < nslot ? ll_load(rl + s) : 0ull;
+    for (int spin = 0; ok && __builtin_amdgcn_ballot_w64(s < nslot && (ll_stale(mr, epoch) || ll_stale(lr, epoch))) != 0; ++spin) {
+      if (spin >= MERGE_SPIN_LIMIT) { ok = false; break; }
+      __builtin_amdgcn_s_sleep(1);
+      if (s < nslot && ll_stale(mr, epoch)) mr = ll_load(rm + s);
+      if (s < nslot && ll_stale(lr, epoch)) lr = ll_load(rl + s);
+    }
+    if (s < nslot) { fs[s] = ll_value(mr); ls[s] = ll_value(lr); m = fmaxf(m, ll_value(mr)); }
+  }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
   float l = 0.f;
-#pragma unroll
-  for (int k = 0; k < PER; ++k) {
-    const int s = lane + 64 * k;
-    const float pmv = __uint_as_float(mv[k]);
-    const float f = (s < nslot && pmv != -INFINITY) ? __builtin_amdgcn_exp2f(pmv - m) : 0.f;
-    if (s < nslot) fs[s] = f;
-    l += __uint_as_float(lv[k]) * f;
+  for (int s = lane; s < nslot; s += 64) {      // each lane revisits the slots it wrote
+    const float pmv = fs[s], f = pmv != -INFINITY ? __builtin_amdgcn_exp2f(pmv - m) : 0.f;
+    fs[s] = f; l += ls[s] * f;
   }
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o, 64);
   wave_lds_sync();
-  f32x4v acc = {0.f, 0.f, 0.f, 0.f};
+  float acc = 0.f;
+  for (int s0 = wave; s0 < nslot; s0 += NW * CH) {
+    if (s0 != wave) {
 #pragma unroll
-  for (int k = 0; k < CH; ++k) {
-    const int s = sg + 2 * k; const float f = s < nslot ? fs[s] : 0.f;
+      for (int k = 0; k < CH; ++k) { const int s = s0 + NW * k; v[k] = s < nslot ? ll_load(ra + (long)s * D) : 0ull; }
+    }
+    for (int spin = 0; ok; ++spin) {
+      bool stale = false;
 #pragma unroll
-    for (int c = 0; c < 4; ++c) acc[c] += __uint_as_float(v[k][c]) * f;
-  }
-  for (int s0 = sg + 2 * CH; s0 < nslot; s0 += 2 * CH) {
-    u32x4 w[CH];
+      for (int k = 0; k < CH; ++k) stale |= s0 + NW * k < nslot && ll_stale(v[k], epoch);
+      if (__builtin_amdgcn_ballot_w64(stale) == 0) break;
+      if (spin >= MERGE_SPIN_LIMIT) { ok = false; break; }
+      __builtin_amdgcn_s_sleep(1);
 #pragma unroll
-    for (int k = 0; k < CH; ++k) w[k] = __builtin_amdgcn_raw_buffer_load_b128(ra, ((s0 + 2 * k) * D + dq) * 4, 0, AUX_AGENT_SCOPE);
+      for (int k = 0; k < CH; ++k) { const int s = s0 + NW * k; if (s < nslot && ll_stale(v[k], epoch)) v[k] = ll_load(ra + (long)s * D); }
+    }
 #pragma unroll
     for (int k = 0; k < CH; ++k) {
-      const int s = s0 + 2 * k; const float f = s < nslot ? fs[s] : 0.f;
-#pragma unroll
-      for (int c = 0; c < 4; ++c) acc[c] += __uint_as_float(w[k][c]) * f;
+      const int s = s0 + NW * k;
+      if (s < nslot) { const float f = fs[s]; acc += f != 0.f ? ll_value(v[k]) * f : 0.f; }      // an empty partial's accumulator may hold anything
     }
   }
+  X.part[wave][lane] = acc;
+  if (lane == 0) X.ok[wave] = ok;
+  lds_barrier();
+  if (wave == 0) {
 #pragma unroll
-  for (int c = 0; c < 4; ++c) acc[c] += __shfl_xor(acc[c], 32, 64);
-  if (sg == 0) {
-    const float inv = l > 0.f ? 1.f / l : 0.f;
-    u32x2 o = {pack_bf16x2(acc[0] * inv, acc[1] * inv), pack_bf16x2(acc[2] * inv, acc[3] * inv)};
-    *reinterpret_cast<u32x2*>(A.out + row * D + dq) = o;
+    for (int w = 1; w < NW; ++w) { acc += X.part[w][lane]; ok = ok && X.ok[w]; }
+    const float o = ok ? (l > 0.f ? acc / l : 0.f) : __builtin_nanf("");
+    A.out[row * D + d] = __builtin_bit_cast(u16, (__bf16)o);
   }
+  lds_barrier();      // part is free for the block's next item
 }
-// Called by all threads of a block (NW waves) after its partial has been written with store_partial().
-// fs: NW x MAX_SLOTS floats of LDS that nothing else uses any more.
+// The merge of a head is shared by its last `mergers` blocks in index order (merge_ranks): the block of rank j takes the half heads
+// j, j + mergers, ..., so that no single CU has to pull all the records.  Called by all threads of a merging block after its own
+// partial has been stored and every thread is done with the LDS that X aliases.
+__device__ __forceinline__ int merge_ranks(int G, int nslot) { return min(min(8, 2 * G), nslot); }
 template <int NW>
-__device__ __forceinline__ void publish_and_merge(const AttnArgs& A, int bh, long qh0, int G, int tid, float* __restrict__ fs) {
-  __shared__ int last;
-  if (!A.tickets) return;
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");      // this thread's write-through stores have reached device scope
-  __syncthreads();
-  if (tid == 0) last = atomicAdd(&A.tickets[bh], 1) == A.nslot - 1;
-  __syncthreads();
-  if (!last) return;
+__device__ __forceinline__ void merge_heads(const AttnArgs& A, long qh0, int G, u32 epoch, int rank, int mergers, int tid, MergeScratch<NW>& X) {
   const int wave = tid >> 6, lane = tid & 63;
-  for (int g = wave; g < G; g += NW) merge_head_by_wave(A, qh0 + g, fs + wave * MAX_SLOTS, lane);
-  if (tid == 0) __hip_atomic_store(&A.tickets[bh], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);      // re-arm for the next launch
+  for (int item = rank; item < 2 * G; item += mergers) merge_half_head<NW>(A, qh0 + (item >> 1), item & 1, epoch, X, wave, lane);
+  // the last block of the grid advances the epoch word for the next launch (the blocks of this launch have read it long ago: they
+  // all started before this block did)
+  if (blockIdx.x == gridDim.x - 1 && tid == 0) __hip_atomic_store(A.epochs, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---------------------------------------------------------------------------------------------------- uncompressed rows
@@ -285,7 +328,8 @@ struct AttnLds {
 // Block merge: one partial per wave plus one (index NW) for the uncompressed rows.  acc[0..3] double as RawScratch before the waves
 // publish, acc[0..NW-1] as the merge factors afterwards.
 template <int NW> struct MergeLds { float m[NW + 1][GMAX], l[NW + 1][GMAX]; float acc[NW + 1][GMAX][D]; };
-static_assert(sizeof(RawScratch) <= 4 * GMAX * D * sizeof(float) && MAX_SLOTS <= GMAX * D, "scratch views must fit the merge buffer");
+static_assert(sizeof(RawScratch) <= 4 * GMAX * D * sizeof(float) && sizeof(MergeScratch<4>) <= 5 * GMAX * D * sizeof(float) &&
+              sizeof(MergeScratch<8>) <= 9 * GMAX * D * sizeof(float), "scratch views must fit the merge buffer");
 struct TableRegs { u32 b0, b1; u32 qlo[4], qhi[4]; };      // one thread's raw inputs of the per-block tables
 // Global loads only, in two parts so that each can be issued as soon as its address is known (the query rows need the batch row, the
 // base rows the cache head) and waited for only when the tables are written.
@@ -567,7 +611,8 @@ __device__ __forceinline__ int uniform_tile(int v) { return __builtin_amdgcn_rea
 
 // ---------------------------------------------------------------------------------------------------- main kernel
 // NW = waves per block: 4 (two blocks per CU) or 8 (one block per CU: half as many partials to merge for the same occupancy)
-template <bool PAGED, int NW>
+// HOST_LEN: the compressed length of every addressed head is the kernel argument S_all (not read from memory)
+template <bool PAGED, int NW, bool HOST_LEN>
 __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const AttnArgs A) {
   constexpr int NT = 64 * NW;
   // one LDS object so that the tables the tile loop reads sit at the lowest addresses (immediate offsets of the LDS loads)
@@ -623,8 +668,12 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
   int S, TLh = 0; long khs = 0, vhs = 0;
   if (PAGED) S = S_ranked >= 0 ? S_ranked : max(A.sl[b], 0);
   else {
-    S = A.sl[ch]; khs = A.k.head_start[ch]; vhs = A.v.head_start[ch];
-    TLh = (A.kt ? A.tl : A.sl)[ch];            // no branch between the loads of this level
+    // lengths known to the host (a Page) come as a kernel argument: the tile range, and with it the first payload loads, then depend on
+    // nothing but the arguments
+    khs = A.k.head_start[ch]; vhs = A.v.head_start[ch];
+    TLh = (A.kt ? A.tl : A.k.head_start)[ch];      // no branch between the loads of this level
+    if (HOST_LEN) S = A.S_all;
+    else S = A.sl[ch];
     if (slot < 0) S = 0;
     if (slot < 0 || !A.kt) TLh = 0;
   }
@@ -672,6 +721,8 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
     load_tags<PAGED>(B, TT, TILE(min(iB, icl)), a, Tg);
   }
   if (tid == 0) next_tile = 2 * NW;
+  // this launch's epoch of the fused merge: one more load of the start-up batch, its value is needed when the block is done
+  const u32 epoch = load_epoch(A, bh);
   GAAC_STAMP(6);
   if (tid < 256) tables_store(L, Tr, tid, G);
   GAAC_STAMP(7);
@@ -768,7 +819,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
   const float m_run = st.m_run == -INFINITY ? -INFINITY : st.mu_run;     // partial maxima are stored in the base-2 domain
   f32x4 (&acc)[8] = st.acc;
 
-  // ---- merge the 4 waves of the block, write the split's partial
+  // ---- merge the waves of the block, write the split's partial
   if (a < G) {
     if (q == 0) { M.m[wave][a] = m_run; M.l[wave][a] = l_run; }
 #pragma unroll
@@ -777,6 +828,8 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
       for (int r = 0; r < 4; ++r) M.acc[wave][a][chan_v(8 * (4 * q + r) + i)] = acc[i][r];
   }
   __syncthreads();
+  const bool fused = A.epochs != nullptr;
+  const int mergers = merge_ranks(G, A.nslot), rank = (int)blockIdx.x % A.nsplit - (A.nsplit - mergers);      // the head's last blocks to start
   const int d = tid & 127;
   for (int g = tid >> 7; g < G; g += NT / 128) {
     float Mx = -INFINITY;
@@ -790,11 +843,21 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
       Lc += M.l[w][g] * f; Ac += live ? M.acc[w][g][d] * f : 0.f;
     }
     const long pidx = (qh0 + g) * A.nslot + split;
-    if (d == 0) { store_partial(A.pm + pidx, Mx); store_partial(A.pl + pidx, Lc); }
-    store_partial(A.pa + pidx * D + d, Ac);
+    if (!fused) {
+      if (d == 0) { store_partial(A.pm + pidx, Mx); store_partial(A.pl + pidx, Lc); }
+      store_partial(A.pa + pidx * D + d, Ac);
+    } else if (A.nslot == 1) {      // the only partial of its rows: it is the result
+      A.out[(qh0 + g) * D + d] = __builtin_bit_cast(u16, (__bf16)(Lc > 0.f ? Ac / Lc : 0.f));
+    } else {
+      if (d == 0) { ll_store(reinterpret_cast<u64*>(A.pm) + pidx, Mx, epoch); ll_store(reinterpret_cast<u64*>(A.pl) + pidx, Lc, epoch); }
+      ll_store(reinterpret_cast<u64*>(A.pa) + pidx * D + d, Ac, epoch);
+    }
   }
   GAAC_STAMP(4);
-  publish_and_merge<NW>(A, bh, qh0, G, tid, &M.acc[0][0][0]);
+  if (fused && rank >= 0 && A.nslot > 1) {
+    lds_barrier();      // every thread is done with the block-merge buffer, which becomes the mergers' scratch
+    merge_heads<NW>(A, qh0, G, epoch, rank, mergers, tid, *reinterpret_cast<MergeScratch<NW>*>(&M.acc[0][0][0]));
+  }
   GAAC_STAMP(5);
 }
 
@@ -892,10 +955,10 @@ __device__ __forceinline__ void consume_raw_tile(const RawTile& R, WaveState& st
   }
 }
 
-struct Bf16Lds { u32x4 qw[GMAX][NG]; float m[4][GMAX], l[4][GMAX]; float acc[4][GMAX][D]; };
+struct Bf16Lds { u32x4 qw[GMAX][NG]; float m[4][GMAX], l[4][GMAX]; float acc[5][GMAX][D]; };      // acc: also the mergers' scratch
 __global__ void __launch_bounds__(256, 2) k_bf16_attn_split(const AttnArgs A) {
   __shared__ Bf16Lds L;
-  const int bh = blockIdx.x, split = blockIdx.y, tid = threadIdx.x;
+  const int bh = (int)blockIdx.x / A.nsplit, split = (int)blockIdx.x % A.nsplit, tid = threadIdx.x;      // a head's blocks are consecutive
   const int b = bh / A.n_kv, kvh = bh % A.n_kv, G = A.G;
   const long qh0 = (long)b * A.n_q + (long)kvh * G;
   const int S = A.sl ? min(max(A.sl[b], 0), A.tcap) : A.tcap;      // per-row lengths on the device (decode steps inside a graph) or one length
@@ -911,6 +974,7 @@ __global__ void __launch_bounds__(256, 2) k_bf16_attn_split(const AttnArgs A) {
   RawTile R0, R1;
   if (tA < thd) load_raw_tile(kh, vh, tA, S, a, q, R0);
   if (tid == 0) next_tile = tlo + 8;
+  const u32 epoch = load_epoch(A, bh);
   // Q as the B operand: lane (head a, quad q), product j covers channels 32 j + 8 q .. + 8 (rows >= G are zero)
   for (int i = tid; i < GMAX * NG; i += 256) {
     const int h = i >> 4, c = i & 15;
@@ -952,6 +1016,7 @@ __global__ void __launch_bounds__(256, 2) k_bf16_attn_split(const AttnArgs A) {
       for (int r = 0; r < 4; ++r) L.acc[wave][a][8 * (4 * q + r) + i] = st.acc[i][r];
   }
   __syncthreads();
+  const int mergers = merge_ranks(G, A.nslot), rank = split - (A.nsplit - mergers);
   const int d = tid & 127;
   for (int g = tid >> 7; g < G; g += 2) {
     float M = -INFINITY;
@@ -964,10 +1029,16 @@ __global__ void __launch_bounds__(256, 2) k_bf16_attn_split(const AttnArgs A) {
       Lc += L.l[w][g] * f; Ac += L.acc[w][g][d] * f;
     }
     const long pidx = (qh0 + g) * A.nslot + split;
-    if (d == 0) { store_partial(A.pm + pidx, M); store_partial(A.pl + pidx, Lc); }
-    store_partial(A.pa + pidx * D + d, Ac);
+    if (A.nslot == 1) A.out[(qh0 + g) * D + d] = __builtin_bit_cast(u16, (__bf16)(Lc > 0.f ? Ac / Lc : 0.f));
+    else {
+      if (d == 0) { ll_store(reinterpret_cast<u64*>(A.pm) + pidx, M, epoch); ll_store(reinterpret_cast<u64*>(A.pl) + pidx, Lc, epoch); }
+      ll_store(reinterpret_cast<u64*>(A.pa) + pidx * D + d, Ac, epoch);
+    }
   }
-  publish_and_merge<4>(A, bh, qh0, G, tid, &L.acc[0][0][0]);
+  if (rank >= 0 && A.nslot > 1) {
+    lds_barrier();
+    merge_heads<4>(A, qh0, G, epoch, rank, mergers, tid, *reinterpret_cast<MergeScratch<4>*>(&L.acc[0][0][0]));
+  }
 }
 
 }  // namespace gaac
@@ -982,10 +1053,11 @@ static int attn_split_impl(
     const uint8_t* smk, const uint8_t* ck, const int* fk, const int* tok, const uint8_t* ovk, const int* ohsk, const uint8_t* b3k, const uint8_t* b4k,
     const uint8_t* smv, const uint8_t* cv, const int* fv, const int* tov, const uint8_t* ovv, const int* ohsv, const uint8_t* b3v, const uint8_t* b4v,
     const void* q, const int* slot, int B, int n_q, int n_kv, const int* SL, int S_pad, float scale, int nsplit, int NB,
-    const void* kt, const void* vt, const int* TL, int TCAP, float* pm, float* pl, float* pa, int* tickets, void* out, void* stream) {
+    const void* kt, const void* vt, const int* TL, int TCAP, void* pm, void* pl, void* pa, unsigned int* epoch, void* out, int S_all, void* stream) {
   GAAC_REQUIRE(n_kv > 0 && n_q > 0 && n_q % n_kv == 0 && n_q / n_kv >= 1 && n_q / n_kv <= GMAX, "GQA group size must be 1..%d (n_q=%d, n_kv=%d)", GMAX, n_q, n_kv);
   GAAC_REQUIRE(smk && ck && fk && tok && ovk && ohsk && b3k && b4k && smv && cv && fv && tov && ovv && ohsv && b3v && b4v, "gaac_attn: null store pointer");
-  GAAC_REQUIRE(q && SL && pm && pl && pa, "gaac_attn: null pointer");
+  GAAC_REQUIRE(q && (SL || S_all >= 0) && pm && pl && pa, "gaac_attn: null pointer");
+  GAAC_REQUIRE(S_all <= S_pad, "gaac_attn: S_all %d exceeds the token stride %d", S_all, S_pad);
   GAAC_REQUIRE(B > 0 && S_pad > 0 && S_pad % T == 0 && NB > 0, "gaac_attn: bad sizes B=%d S_pad=%d NB=%d", B, S_pad, NB);
   const bool has_tail = kt != nullptr;
   GAAC_REQUIRE(!has_tail || (vt && TL && TCAP >= 1 && TCAP <= T), "gaac_attn: tail needs kt, vt, TL and 1 <= TCAP <= %d", T);
@@ -995,19 +1067,23 @@ static int attn_split_impl(
   AttnArgs A;
   A.k = StoreView{smk, ck, fk, tok, ovk, ohsk, b3k, b4k};
   A.v = StoreView{smv, cv, fv, tov, ovv, ohsv, b3v, b4v};
-  A.q = (const u16*)q; A.pm = pm; A.pl = pl; A.pa = pa; A.slot = slot; A.sl = SL;
+  A.q = (const u16*)q; A.pm = (float*)pm; A.pl = (float*)pl; A.pa = (float*)pa; A.slot = slot; A.sl = SL; A.S_all = S_all < 0 ? -1 : S_all;
   A.S_pad = S_pad; A.scale_log2e = scale * 1.4426950408889634f; A.nsplit = nsplit; A.nslot = nslot;
   A.n_kv = n_kv; A.n_q = n_q; A.G = n_q / n_kv; A.NB = NB;
   A.kt = (const u16*)kt; A.vt = (const u16*)vt; A.tl = TL; A.tcap = TCAP;
-  A.tickets = tickets; A.out = (u16*)out;
-  GAAC_REQUIRE(!tickets || out, "gaac_attn: the fused merge needs an output buffer");
+  A.epochs = epoch; A.out = (u16*)out;
+  GAAC_REQUIRE(!epoch || out, "gaac_attn: the fused merge needs an output buffer");
   A.pool = nullptr; A.raw = nullptr; A.mt = nullptr; A.bt = nullptr; A.bt_stride = 0; A.TS = 0;
 #ifdef GAAC_PHASE_TIMING
   A.dbg = g_dbg;
 #endif
   // few blocks: one 8-wave block per CU (half as many partials); otherwise two 4-wave blocks per CU
-  if ((long)B * n_kv * nslot <= 256) hipLaunchKernelGGL((k_attn_split<false, 8>), dim3(B * n_kv * nslot), dim3(512), 0, (hipStream_t)stream, A);
-  else hipLaunchKernelGGL((k_attn_split<false, 4>), dim3(B * n_kv * nslot), dim3(256), 0, (hipStream_t)stream, A);
+  const bool wide = (long)B * n_kv * nslot <= 256;
+  const dim3 grid(B * n_kv * nslot), block(wide ? 512 : 256);
+  if (wide && S_all >= 0) hipLaunchKernelGGL((k_attn_split<false, 8, true>), grid, block, 0, (hipStream_t)stream, A);
+  else if (wide) hipLaunchKernelGGL((k_attn_split<false, 8, false>), grid, block, 0, (hipStream_t)stream, A);
+  else if (S_all >= 0) hipLaunchKernelGGL((k_attn_split<false, 4, true>), grid, block, 0, (hipStream_t)stream, A);
+  else hipLaunchKernelGGL((k_attn_split<false, 4, false>), grid, block, 0, (hipStream_t)stream, A);
   return launch_status("gaac_attn(split)");
 }
 
@@ -1017,7 +1093,7 @@ extern "C" int gaac_attn_split(
     const void* q, const int* slot, int B, int n_q, int n_kv, const int* SL, int S_pad, float scale, int nsplit, int NB,
     const void* kt, const void* vt, const int* TL, int TCAP, float* pm, float* pl, float* pa, void* stream) {
   return attn_split_impl(smk, ck, fk, tok, ovk, ohsk, b3k, b4k, smv, cv, fv, tov, ovv, ohsv, b3v, b4v, q, slot, B, n_q, n_kv, SL, S_pad,
-                         scale, nsplit, NB, kt, vt, TL, TCAP, pm, pl, pa, nullptr, nullptr, stream);
+                         scale, nsplit, NB, kt, vt, TL, TCAP, pm, pl, pa, nullptr, nullptr, -1, stream);
 }
 
 extern "C" int gaac_attn_combine(const float* pm, const float* pl, const float* pa, void* out, int n_rows, int nslot, void* stream) {
@@ -1034,7 +1110,7 @@ extern "C" int gaac_attn_launch(
     float* pm, float* pl, float* pa, void* out, void* stream) {
   GAAC_REQUIRE(out, "gaac_attn_launch: null output");
   int rc = attn_split_impl(smk, ck, fk, tok, ovk, ohsk, b3k, b4k, smv, cv, fv, tov, ovv, ohsv, b3v, b4v, q, slot, B, n_q, n_kv, SL, S_pad,
-                           scale, nsplit, NB, kt, vt, TL, TCAP, pm, pl, pa, nullptr, nullptr, stream);
+                           scale, nsplit, NB, kt, vt, TL, TCAP, pm, pl, pa, nullptr, nullptr, -1, stream);
   if (rc) return rc;
   return gaac_attn_combine(pm, pl, pa, out, B * n_q, nsplit, stream);
 }
@@ -1043,20 +1119,20 @@ extern "C" int gaac_attn_fused(
     const uint8_t* smk, const uint8_t* ck, const int* fk, const int* tok, const uint8_t* ovk, const int* ohsk, const uint8_t* b3k, const uint8_t* b4k,
     const uint8_t* smv, const uint8_t* cv, const int* fv, const int* tov, const uint8_t* ovv, const int* ohsv, const uint8_t* b3v, const uint8_t* b4v,
     const void* q, const int* slot, int B, int n_q, int n_kv, const int* SL, int S_pad, float scale, int nsplit, int NB,
-    const void* kt, const void* vt, const int* TL, int TCAP,
-    float* pm, float* pl, float* pa, int* tickets, void* out, void* stream) {
-  GAAC_REQUIRE(out && tickets, "gaac_attn_fused: null output or ticket buffer");
+    const void* kt, const void* vt, const int* TL, int TCAP, int S_all,
+    unsigned long long* pm, unsigned long long* pl, unsigned long long* pa, unsigned int* epoch, void* out, void* stream) {
+  GAAC_REQUIRE(out && epoch, "gaac_attn_fused: null output or epoch buffer");
   return attn_split_impl(smk, ck, fk, tok, ovk, ohsk, b3k, b4k, smv, cv, fv, tov, ovv, ohsv, b3v, b4v, q, slot, B, n_q, n_kv, SL, S_pad,
-                         scale, nsplit, NB, kt, vt, TL, TCAP, pm, pl, pa, tickets, out, stream);
+                         scale, nsplit, NB, kt, vt, TL, TCAP, pm, pl, pa, epoch, out, S_all, stream);
 }
 
 extern "C" int gaac_paged_attn(
     const uint8_t* pool, int TS, const void* raw, const int* mt, const int* bt, int bt_stride, const int* seq_lens, int max_seq_len,
     const void* q, int B, int n_q, int n_kv, float scale, int nsplit,
     const uint8_t* b3k, const uint8_t* b4k, const uint8_t* b3v, const uint8_t* b4v, int NB,
-    float* pm, float* pl, float* pa, int* tickets, void* out, void* stream) {
+    unsigned long long* pm, unsigned long long* pl, unsigned long long* pa, unsigned int* epoch, void* out, void* stream) {
   GAAC_REQUIRE(n_kv > 0 && n_q > 0 && n_q % n_kv == 0 && n_q / n_kv <= GMAX, "GQA group size must be 1..%d (n_q=%d, n_kv=%d)", GMAX, n_q, n_kv);
-  GAAC_REQUIRE(pool && raw && mt && bt && seq_lens && q && b3k && b4k && b3v && b4v && pm && pl && pa && tickets && out, "gaac_paged_attn: null pointer");
+  GAAC_REQUIRE(pool && raw && mt && bt && seq_lens && q && b3k && b4k && b3v && b4v && pm && pl && pa && epoch && out, "gaac_paged_attn: null pointer");
   GAAC_REQUIRE(B > 0 && NB > 0 && TS >= SLOT_OV && TS % 16 == 0 && bt_stride > 0, "gaac_paged_attn: bad sizes B=%d NB=%d TS=%d", B, NB, TS);
   GAAC_REQUIRE(nsplit >= 1 && nsplit <= MAX_SLOTS, "gaac_paged_attn: nsplit must be in 1..%d", MAX_SLOTS);
   const long max_tiles = ((long)max_seq_len + T - 1) / T;
@@ -1065,31 +1141,32 @@ extern "C" int gaac_paged_attn(
   AttnArgs A;
   A.k = StoreView{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, b3k, b4k};
   A.v = StoreView{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, b3v, b4v};
-  A.q = (const u16*)q; A.pm = pm; A.pl = pl; A.pa = pa; A.slot = nullptr; A.sl = seq_lens;
+  A.q = (const u16*)q; A.pm = (float*)pm; A.pl = (float*)pl; A.pa = (float*)pa; A.slot = nullptr; A.sl = seq_lens; A.S_all = -1;
   A.S_pad = 0; A.scale_log2e = scale * 1.4426950408889634f; A.nsplit = nsplit; A.nslot = nsplit;
   A.n_kv = n_kv; A.n_q = n_q; A.G = n_q / n_kv; A.NB = NB;
   A.kt = nullptr; A.vt = nullptr; A.tl = nullptr; A.tcap = 0;
-  A.tickets = tickets; A.out = (u16*)out;
+  A.epochs = epoch; A.out = (u16*)out;
   A.pool = pool; A.raw = (const u16*)raw; A.mt = mt; A.bt = bt; A.bt_stride = bt_stride; A.TS = TS;
 #ifdef GAAC_PHASE_TIMING
   A.dbg = g_dbg;
 #endif
-  if ((long)B * n_kv * nsplit <= 256) hipLaunchKernelGGL((k_attn_split<true, 8>), dim3(B * n_kv * nsplit), dim3(512), 0, (hipStream_t)stream, A);
-  else hipLaunchKernelGGL((k_attn_split<true, 4>), dim3(B * n_kv * nsplit), dim3(256), 0, (hipStream_t)stream, A);
+  if ((long)B * n_kv * nsplit <= 256) hipLaunchKernelGGL((k_attn_split<true, 8, false>), dim3(B * n_kv * nsplit), dim3(512), 0, (hipStream_t)stream, A);
+  else hipLaunchKernelGGL((k_attn_split<true, 4, false>), dim3(B * n_kv * nsplit), dim3(256), 0, (hipStream_t)stream, A);
   return launch_status("gaac_paged_attn");
 }
 
 extern "C" int gaac_bf16_attn(const void* k, const void* v, int S, const int* seq_lens, long head_stride_tokens, const void* q, int B, int n_q,
-                              int n_kv, float scale, int nsplit, float* pm, float* pl, float* pa, int* tickets, void* out, void* stream) {
+                              int n_kv, float scale, int nsplit, unsigned long long* pm, unsigned long long* pl, unsigned long long* pa,
+                              unsigned int* epoch, void* out, void* stream) {
   GAAC_REQUIRE(n_kv > 0 && n_q > 0 && n_q % n_kv == 0 && n_q / n_kv <= GMAX, "GQA group size must be 1..%d (n_q=%d, n_kv=%d)", GMAX, n_q, n_kv);
-  GAAC_REQUIRE(k && v && q && pm && pl && pa && tickets && out, "gaac_bf16_attn: null pointer");
+  GAAC_REQUIRE(k && v && q && pm && pl && pa && epoch && out, "gaac_bf16_attn: null pointer");
   GAAC_REQUIRE(B > 0 && S > 0 && head_stride_tokens >= S && nsplit >= 1 && nsplit <= MAX_SLOTS, "gaac_bf16_attn: bad sizes");
   AttnArgs A = {};
-  A.q = (const u16*)q; A.pm = pm; A.pl = pl; A.pa = pa;
+  A.q = (const u16*)q; A.pm = (float*)pm; A.pl = (float*)pl; A.pa = (float*)pa; A.S_all = -1;
   A.S_pad = (int)head_stride_tokens; A.scale_log2e = scale * 1.4426950408889634f; A.nsplit = nsplit; A.nslot = nsplit;
   A.n_kv = n_kv; A.n_q = n_q; A.G = n_q / n_kv; A.NB = 1;
   A.kt = (const u16*)k; A.vt = (const u16*)v; A.tcap = S; A.sl = seq_lens;
-  A.tickets = tickets; A.out = (u16*)out;
-  hipLaunchKernelGGL(k_bf16_attn_split, dim3(B * n_kv, nsplit), dim3(256), 0, (hipStream_t)stream, A);
+  A.epochs = epoch; A.out = (u16*)out;
+  hipLaunchKernelGGL(k_bf16_attn_split, dim3(B * n_kv * nsplit), dim3(256), 0, (hipStream_t)stream, A);
   return launch_status("gaac_bf16_attn");
 }

@@ -26,15 +26,34 @@ def choose_nsplit(B: int, n_kv: int, S: int, target_ctas: int = 256, min_tok: in
 
 
 class AttnWorkspace:
-    """Output + split partials of one launch shape (fp32 m, l [rows*NSLOT] and acc [rows*NSLOT*D]; rows = B*n_q)."""
+    """Output + split partials of one launch shape (rows = B*n_q): m, l [rows*NSLOT] and acc [rows*NSLOT*D].  The one-kernel launch
+    stores every partial value as a 64-bit record (fp32 bits | launch epoch << 32); the two-kernel launch writes plain fp32 into the
+    front of the same buffers.  epoch: one word, the epoch of the last merged one-kernel launch on this workspace."""
     def __init__(self, rows: int, nslot: int, dtype, dev, with_out: bool = True):
         self.rows, self.nslot = rows, nslot
         self.out = torch.empty(rows, D, dtype=dtype, device=dev) if with_out else None      # None: a fresh output per launch
-        self.pm = torch.empty(rows * nslot, dtype=torch.float32, device=dev)
-        self.pl = torch.empty(rows * nslot, dtype=torch.float32, device=dev)
-        self.pa = torch.empty(rows * nslot * D, dtype=torch.float32, device=dev)
-        # arrival counters of the fused merge, one per (batch row, kv head) (at most `rows` of them); every launch leaves them zero
-        self.tickets = torch.zeros(rows, dtype=torch.int32, device=dev)
+        self.pm = torch.zeros(rows * nslot, dtype=torch.int64, device=dev)
+        self.pl = torch.zeros(rows * nslot, dtype=torch.int64, device=dev)
+        self.pa = torch.zeros(rows * nslot * D, dtype=torch.int64, device=dev)
+        self.epoch = torch.zeros(1, dtype=torch.int32, device=dev)
+
+    def reset(self):
+        """Re-arm after a failed launch: the epochs and the records start from zero again."""
+        for t in (self.pm, self.pl, self.pa, self.epoch): t.zero_()
+
+
+_shared_ws: dict = {}
+
+
+def shared_workspace(rows: int, nslot: int, dtype, dev) -> AttnWorkspace:
+    """The workspace that callers who pass none share: one per (device, launch shape, stream), zeroed once when it is made (a fresh
+    buffer per call would have to be cleared per call: recycled memory may hold records whose epoch matches a new counter).
+    It has no output buffer of its own, so every launch returns a fresh tensor."""
+    dev = torch.device(dev)
+    key = (dev.type, dev.index if dev.index is not None else torch.cuda.current_device(), rows, nslot, dtype, torch.cuda.current_stream(dev).cuda_stream)
+    ws = _shared_ws.get(key)
+    if ws is None: ws = _shared_ws[key] = AttnWorkspace(rows, nslot, dtype, dev, with_out=False)
+    return ws
 
 
 def _store_args(st):
@@ -43,10 +62,11 @@ def _store_args(st):
     return (p(st.sm), p(st.codes), p(st.flags), p(st.tile_off), p(st.ovf), p(hs), p(st.base3), p(st.base4))
 
 
-def attn_launch(K, V, q2d, slots, n_q, n_kv, SL, S_pad, scale, nsplit, kt=None, vt=None, TL=None, TCAP=0, ws=None, phase="fused"):
+def attn_launch(K, V, q2d, slots, n_q, n_kv, SL, S_pad, scale, nsplit, kt=None, vt=None, TL=None, TCAP=0, ws=None, phase="fused", S_all=-1):
     """K, V: objects with sm, codes, flags, tile_off, ovf, head_start|ovf_head_start, base3, base4 (a Page or a cache store).
-    q2d: [B*n_q, D] bf16 contiguous.  Returns [B*n_q, D] bf16.  phase: "fused" (one kernel, the last block of each
-    kv head merges) | "both" (split kernel then merge kernel) | "split" | "combine" (the halves of "both")."""
+    q2d: [B*n_q, D] bf16 contiguous.  Returns [B*n_q, D] bf16.  phase: "fused" (one kernel, one block of each
+    kv head merges) | "both" (split kernel then merge kernel) | "split" | "combine" (the halves of "both").
+    S_all >= 0: every addressed head holds exactly S_all compressed tokens (SL is not read by the one-kernel launch)."""
     G = n_q // max(1, n_kv)
     if not (1 <= G <= GMAX and G * n_kv == n_q):
         raise RuntimeError(f"GQA group size must be 1..{GMAX}")
@@ -56,7 +76,7 @@ def attn_launch(K, V, q2d, slots, n_q, n_kv, SL, S_pad, scale, nsplit, kt=None, 
     has_tail = kt is not None and kt.numel() > 0
     nslot = nsplit        # the raw tail is folded into the last split's partial
     if ws is None:
-        ws = AttnWorkspace(B * n_q, nslot, q2d.dtype, q2d.device)
+        ws = shared_workspace(B * n_q, nslot, q2d.dtype, q2d.device)
     elif ws.rows != B * n_q or ws.nslot != nslot:
         raise RuntimeError("attention workspace does not match the launch shape")
     p = _lib.ptr
@@ -65,11 +85,12 @@ def attn_launch(K, V, q2d, slots, n_q, n_kv, SL, S_pad, scale, nsplit, kt=None, 
         _lib.call("gaac_attn_combine", p(ws.pm), p(ws.pl), p(ws.pa), p(out), B * n_q, nslot, _lib.stream())
         return out
     args = (*_store_args(K), *_store_args(V), p(q2d), p(slots), B, n_q, n_kv, p(SL), S_pad, float(scale), nsplit, K.base3.shape[0],
-            p(kt) if has_tail else None, p(vt) if has_tail else None, p(TL) if has_tail else None, TCAP if has_tail else 0,
-            p(ws.pm), p(ws.pl), p(ws.pa))
+            p(kt) if has_tail else None, p(vt) if has_tail else None, p(TL) if has_tail else None, TCAP if has_tail else 0)
     if phase == "fused":
-        _lib.call("gaac_attn_fused", *args, p(ws.tickets), p(out), _lib.stream())
-    elif phase == "split":
+        _lib.call("gaac_attn_fused", *args, int(S_all), p(ws.pm), p(ws.pl), p(ws.pa), p(ws.epoch), p(out), _lib.stream())
+        return out
+    args = (*args, p(ws.pm), p(ws.pl), p(ws.pa))
+    if phase == "split":
         _lib.call("gaac_attn_split", *args, _lib.stream())
     else:
         _lib.call("gaac_attn_launch", *args, p(out), _lib.stream())
@@ -85,7 +106,7 @@ def attention(q, kp, vp, scale=None, nsplit=None, phase="fused"):
     if nsplit is None: nsplit = choose_nsplit(B, n_kv, kp.S)
     SL = torch.full((kp.H,), kp.S, dtype=torch.int32, device=dev)
     out = attn_launch(kp, vp, q.reshape(B * n_q, Dq).contiguous(), None, n_q, n_kv, SL, kp.sm.shape[1] // D,
-                      scale if scale is not None else Dq ** -0.5, nsplit, phase=phase)
+                      scale if scale is not None else Dq ** -0.5, nsplit, phase=phase, S_all=kp.S)
     return out.view(B, n_q, Dq)
 
 
@@ -98,9 +119,10 @@ def bf16_attention(q, k, v, scale=None, nsplit=None, ws=None, seq_lens=None, out
     n_kv = H // B
     if k.stride(1) != D or v.stride(1) != D or k.stride(0) != v.stride(0): raise RuntimeError("bf16_attention expects token rows of 128 contiguous elements")
     if nsplit is None: nsplit = choose_nsplit(B, n_kv, S)
-    if ws is None: ws = AttnWorkspace(B * n_q, nsplit, q.dtype, q.device, with_out=out is None)
+    if ws is None: ws = shared_workspace(B * n_q, nsplit, q.dtype, q.device)
+    elif ws.rows != B * n_q or ws.nslot != nsplit: raise RuntimeError("attention workspace does not match the launch shape")
     if out is None: out = ws.out if ws.out is not None else torch.empty(B * n_q, D, dtype=q.dtype, device=q.device)
     p = _lib.ptr
     _lib.call("gaac_bf16_attn", p(k), p(v), S, p(seq_lens), k.stride(0) // D, p(q.contiguous()), B, n_q, n_kv,
-              float(scale if scale is not None else Dq ** -0.5), nsplit, p(ws.pm), p(ws.pl), p(ws.pa), p(ws.tickets), p(out), _lib.stream())
+              float(scale if scale is not None else Dq ** -0.5), nsplit, p(ws.pm), p(ws.pl), p(ws.pa), p(ws.epoch), p(out), _lib.stream())
     return out.view(B, n_q, Dq)

@@ -97,7 +97,7 @@ class CompressedKVCache:
         # set by the append kernel instead of writing out of bounds: bit 0 = a head was full, bit 1 = an escape stream was full
         self.overflow = torch.zeros(1, dtype=torch.int32, device=device)
         self.growable = True       # set False once graphs captured the buffer addresses
-        self._partials = {}        # split partials + merge tickets per launch shape (stable addresses for graph replays)
+        self._partials = {}        # split partials + merge epochs per launch shape (stable addresses for graph replays)
 
     @staticmethod
     def bytes_per_slot(n_kv: int, capacity: int, ovf_bytes_per_tile: int = 128, per_sequence_bases: bool = True) -> int:

@@ -9,7 +9,7 @@ from __future__ import annotations
 import numpy as np
 import torch
 from . import _lib
-from .kernel import AttnWorkspace
+from .kernel import AttnWorkspace, shared_workspace
 
 D = 128
 BLOCK = 16
@@ -124,11 +124,11 @@ def paged_attention(q, out, buf, raw, mt, bt, seq_lens, bases, TS, n_q, n_kv, ns
     B = q.shape[0]
     if q.shape[-1] != D: raise RuntimeError("head_dim must be 128")
     if max_seq_len is None: max_seq_len = bt.shape[1] * BLOCK
-    if ws is None: ws = AttnWorkspace(B * n_q, nsplit, q.dtype, q.device, with_out=False)
+    if ws is None: ws = shared_workspace(B * n_q, nsplit, q.dtype, q.device)
     elif ws.rows != B * n_q or ws.nslot != nsplit: raise RuntimeError("attention workspace does not match the launch shape")
     p = _lib.ptr
     q = q.contiguous()
     _lib.call("gaac_paged_attn", p(buf), TS, p(raw), p(mt), p(bt), bt.stride(0), p(seq_lens), int(max_seq_len), p(q), B, n_q, n_kv,
               float(1.0 / (D ** 0.5)), nsplit, p(bases[0]), p(bases[1]), p(bases[2]), p(bases[3]), bases[0].shape[0],
-              p(ws.pm), p(ws.pl), p(ws.pa), p(ws.tickets), p(out), _lib.stream())
+              p(ws.pm), p(ws.pl), p(ws.pa), p(ws.epoch), p(out), _lib.stream())
     return out

@@ -75,16 +75,23 @@ int gaac_attn_split(
     const void* kt, const void* vt, const int* TL, int TCAP, float* pm, float* pl, float* pa, void* stream);
 int gaac_attn_combine(const float* pm, const float* pl, const float* pa, void* out, int n_rows, int nslot, void* stream);
 
-/* gaac_attn_launch as ONE kernel: every block publishes its partial and draws a ticket from tickets[b*n_kv + kv head];
- * the block that draws the last one merges the NSLOT partials of its G query heads (gaac_combine, kernel.py:281-294) and
- * resets the counter.  tickets: int32 [B*n_kv], zero before the first launch (each launch leaves it zero); launches that
- * share pm/pl/pa/tickets must be ordered on one stream. */
+/* gaac_attn_launch as ONE kernel: the merge of the NSLOT partials (gaac_combine, kernel.py:281-294) is done inside the split kernel
+ * by the last (up to eight) blocks of each (batch row, kv head) in index order, each taking a share of the head's output, without
+ * atomics.  *epoch holds the epoch of the last merged launch; this launch's epoch is that + 1.  Partials travel as 64-bit records
+ * (fp32 bits | epoch << 32) written and read with single 64-bit accesses, so a merging block recognises the records of this launch
+ * without waiting for an acknowledgement; it re-reads records that have not arrived yet (bounded; rows are written as NaN if they
+ * never do).  The last block of the grid stores the new epoch as its last action.
+ * pm, pl: records [B*n_q*nsplit]; pa: records [B*n_q*nsplit*128]; epoch: one uint32.  Zero epoch, pm, pl and pa before the first
+ * launch and to re-arm them after a failed launch.  Launches of any shape may share them (buffers sized for the largest) as long as
+ * they are ordered on one stream.
+ * S_all >= 0: every cache head the launch addresses holds exactly S_all compressed tokens (a Page: lengths are known to the host);
+ * SL is then not read and may be NULL, which takes one dependent load off the start of every block.  S_all < 0: lengths come from SL. */
 int gaac_attn_fused(
     const uint8_t* smk, const uint8_t* ck, const int* fk, const int* tok, const uint8_t* ovk, const int* ohsk, const uint8_t* b3k, const uint8_t* b4k,
     const uint8_t* smv, const uint8_t* cv, const int* fv, const int* tov, const uint8_t* ovv, const int* ohsv, const uint8_t* b3v, const uint8_t* b4v,
     const void* q, const int* slot, int B, int n_q, int n_kv, const int* SL, int S_pad, float scale, int nsplit, int NB,
-    const void* kt, const void* vt, const int* TL, int TCAP,
-    float* pm, float* pl, float* pa, int* tickets, void* out, void* stream);
+    const void* kt, const void* vt, const int* TL, int TCAP, int S_all,
+    unsigned long long* pm, unsigned long long* pl, unsigned long long* pa, unsigned int* epoch, void* out, void* stream);
 
 /* CompressedKVCache.append, /root/reference/gaac/kv_cache.py:172-181 (kernels _append_one/_append_kv/_advance, :22-96), as one
  * launch: row i = b*n_kv + kvh of k_new/v_new [B, n_kv, 128] bf16 goes to tail row tail_len[h] of cache head
@@ -121,19 +128,21 @@ int gaac_paged_decode(const uint8_t* pool, int TS, const void* raw, const int* m
                       long row_stride, const uint8_t* b3k, const uint8_t* b4k, const uint8_t* b3v, const uint8_t* b4v, int n_kv, void* stream);
 /* paged_attention -> gaac_vpaged_launch, paged_kernel.py:42-277: decode attention of B rows over the pool through the block table
  * bt int32 [B][bt_stride] and the mode table; seq_lens int32 [B] (tokens incl. the filling block; no separate tail); max_seq_len =
- * an upper bound of seq_lens known to the host (bounds the tiles per split, at most 1024).  Partials pm, pl [B*n_q*nsplit],
- * pa [B*n_q*nsplit*128], tickets int32 [B*n_kv] (zero) as in gaac_attn_fused; out bf16 [B*n_q][128]. */
+ * an upper bound of seq_lens known to the host (bounds the tiles per split, at most 1024).  Partial records pm, pl [B*n_q*nsplit],
+ * pa [B*n_q*nsplit*128] and the epoch word as in gaac_attn_fused; out bf16 [B*n_q][128]. */
 int gaac_paged_attn(const uint8_t* pool, int TS, const void* raw, const int* mt, const int* bt, int bt_stride, const int* seq_lens,
                     int max_seq_len, const void* q, int B, int n_q, int n_kv, float scale, int nsplit,
                     const uint8_t* b3k, const uint8_t* b4k, const uint8_t* b3v, const uint8_t* b4v, int NB,
-                    float* pm, float* pl, float* pa, int* tickets, void* out, void* stream);
+                    unsigned long long* pm, unsigned long long* pl, unsigned long long* pa, unsigned int* epoch, void* out,
+                    void* stream);
 
 /* Baseline, not part of the compressed path: decode attention over UNCOMPRESSED bf16 K/V [B*n_kv][head_stride_tokens][128] (S tokens
  * per head, or seq_lens[b] <= S tokens for batch row b when seq_lens != NULL) with the same block / wave / MFMA structure, merge and
  * partial buffers as gaac_attn_fused.  The reference compares against flash-attn (examples/attention.py:29-30); this is the same-GPU
  * counterpart for that comparison. */
 int gaac_bf16_attn(const void* k, const void* v, int S, const int* seq_lens, long head_stride_tokens, const void* q, int B, int n_q,
-                   int n_kv, float scale, int nsplit, float* pm, float* pl, float* pa, int* tickets, void* out, void* stream);
+                   int n_kv, float scale, int nsplit, unsigned long long* pm, unsigned long long* pl, unsigned long long* pa,
+                   unsigned int* epoch, void* out, void* stream);
 
 /* Measurement aid with no counterpart in the reference: a plain copy of nbytes (multiple of 16) with 16-byte accesses per lane,
  * the known-size kernel that HBM traffic counters (FETCH_SIZE / WRITE_SIZE) are scaled against. */

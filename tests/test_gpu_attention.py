@@ -64,24 +64,50 @@ def test_result_does_not_depend_on_the_split_count():
         assert np.abs(o - outs[0]).max() <= 2 ** -7 * np.abs(outs[0]).max()
 
 
-def test_fused_merge_equals_the_two_kernel_launch_and_rearms_its_tickets():
-    """One-kernel launch (last block merges) vs split kernel + merge kernel: same partials, so the outputs agree to the last
-    bf16 bit or one ulp of rounding order; launched three times on one workspace to show the counters reset themselves."""
+def test_fused_merge_equals_the_two_kernel_launch_on_a_reused_workspace():
+    """One-kernel launch (one block of each kv head merges) vs split kernel + merge kernel: same partials, so the outputs agree to the
+    last bf16 bit or one ulp of rounding order.  Launched several times on one workspace, alternating with the two-kernel launch that
+    overwrites the same buffers with plain fp32: the workspace's epoch word counts the merged launches and the epoch in every
+    record keeps launches apart.  reset() re-arms the workspace."""
     dev = require_gpu()
     from gaac_amd.kernel import attn_launch, AttnWorkspace
-    for (B, n_kv, G, S, ns) in [(1, 8, 4, 4096, 16), (2, 2, 16, 1000, 7), (3, 2, 1, 16, 1), (1, 8, 4, 8192, 64)]:
+    for (B, n_kv, G, S, ns) in [(1, 8, 4, 4096, 16), (2, 2, 16, 1000, 7), (3, 2, 1, 16, 1), (1, 8, 4, 8192, 64), (1, 2, 4, 3000, 100)]:
         _, _, kp, vp = _pages(B, n_kv, S, dev)
         n_q = n_kv * G
         q = to_bf16(randn_bf16((B * n_q, 128), seed=9, scale=0.3), dev)
         slots = torch.arange(B, dtype=torch.int32, device=dev)
         SL = torch.full((B * n_kv,), S, dtype=torch.int32, device=dev)
         ws = AttnWorkspace(B * n_q, ns, torch.bfloat16, dev)
-        run = lambda ph: attn_launch(kp, vp, q, slots, n_q, n_kv, SL, kp.sm.shape[1] // 128, SCALE, ns, ws=ws, phase=ph).float().clone()
+        run = lambda ph, **kw: attn_launch(kp, vp, q, slots, n_q, n_kv, SL, kp.sm.shape[1] // 128, SCALE, ns, ws=ws, phase=ph, **kw).float().clone()
         two = run("both")
-        for _ in range(3):
-            one = run("fused")
-            assert (one - two).abs().max().item() <= 2.0 ** -7 * two.abs().max().item()
-        assert int(ws.tickets.abs().sum().item()) == 0
+        n = 0
+        for rnd in range(3):
+            for _ in range(3):
+                one = run("fused", S_all=S if rnd == 1 else -1); n += 1
+                assert (one - two).abs().max().item() <= 2.0 ** -7 * two.abs().max().item()
+            assert int(ws.epoch) == (n if ns > 1 else 0)
+            assert (run("both") - two).abs().max().item() == 0.0
+        ws.reset()
+        assert (run("fused") - two).abs().max().item() <= 2.0 ** -7 * two.abs().max().item()
+        assert int(ws.epoch) == (1 if ns > 1 else 0)
+
+
+def test_launch_shapes_that_share_a_workspace_do_not_mix_their_records():
+    """attention() without a workspace uses one shared per (rows, splits): (1, 8, 4) and (1, 2, 16) at 4096 tokens have the same 32 rows
+    and 16 splits but other kv heads, so each launch finds the other shape's records in the buffers.  The epoch is one word per
+    workspace: whatever an earlier launch wrote is older than the running one."""
+    dev = require_gpu()
+    from gaac_amd import attention
+    cases = []
+    for (n_kv, G, seed) in [(8, 4, 31), (2, 16, 32), (4, 8, 33)]:
+        k16, v16, kp, vp = _pages(1, n_kv, 4096, dev, seed=seed, soft=True)
+        q16 = randn_bf16((1, n_kv * G, 128), seed=seed + 5, scale=1.0)
+        ref = O.ref_attention(q16[0], k16.transpose(1, 0, 2), v16.transpose(1, 0, 2), SCALE)
+        cases.append((to_bf16(q16, dev), kp, vp, ref))
+    for rnd in range(6):
+        for (q, kp, vp, ref) in cases[rnd % 3:] + cases[:rnd % 3]:
+            out = O.bf16_to_f32(to_u16(attention(q, kp, vp, SCALE)))[0]
+            assert np.abs(out - ref).max() <= 2e-2 * np.abs(ref).max() + 1e-3
 
 
 @pytest.mark.parametrize("B,n_kv,G,S", [(1, 8, 4, 4096), (2, 2, 16, 1000), (3, 2, 1, 16), (1, 4, 6, 333)])
