@@ -270,7 +270,10 @@ __device__ __forceinline__ void wave_rows_attend(float (*__restrict__ sc)[T], co
   {
     u32x4 kv[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) kv[j] = t < nvalid ? *reinterpret_cast<const u32x4*>(krows + t * D + 32 * c + 8 * j) : u32x4{0u, 0u, 0u, 0u};
+    for (int j = 0; j < 4; ++j) {      // no load under a branch: rows past the end read the last valid row and are zeroed
+      kv[j] = *reinterpret_cast<const u32x4*>(krows + min(t, nvalid - 1) * D + 32 * c + 8 * j);
+      if (t >= nvalid) kv[j] = u32x4{0u, 0u, 0u, 0u};
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -304,7 +307,9 @@ __device__ __forceinline__ void wave_rows_attend(float (*__restrict__ sc)[T], co
   wave_lds_sync();
   u32 vv[T];
 #pragma unroll
-  for (int tk = 0; tk < T; ++tk) vv[tk] = tk < nvalid ? *reinterpret_cast<const u32*>(vrows + tk * D + 2 * lane) : 0u;
+  for (int tk = 0; tk < T; ++tk) vv[tk] = *reinterpret_cast<const u32*>(vrows + min(tk, nvalid - 1) * D + 2 * lane);
+#pragma unroll
+  for (int tk = 0; tk < T; ++tk) vv[tk] = tk < nvalid ? vv[tk] : 0u;      // rows past the end weigh 0: keep an Inf of the clamped row out of 0 * Inf
   for (int g = 0; g < G; ++g) {
     float a0 = 0.f, a1 = 0.f;
 #pragma unroll
@@ -420,9 +425,9 @@ __device__ __forceinline__ void load_tags(const Bases& B, const TileTable& TT, i
   }
 }
 
+// the tile's sign/mantissa and code bytes (paged mode: the slot index comes with the tags)
 template <bool PAGED>
-__device__ __forceinline__ void load_tile(const Bases& B, int tile, int lane, const TagRegs& Tg, TileRegs& R) {
-  const int q = lane >> 4;
+__device__ __forceinline__ void load_tile_payload(const Bases& B, int tile, int lane, const TagRegs& Tg, TileRegs& R) {
   if (PAGED) {
     const uint8_t* ks = B.kov + (size_t)__builtin_amdgcn_readfirstlane(Tg.kto) * (size_t)B.TS;
     const uint8_t* vs = B.vov + (size_t)__builtin_amdgcn_readfirstlane(Tg.vto) * (size_t)B.TS;
@@ -442,6 +447,11 @@ __device__ __forceinline__ void load_tile(const Bases& B, int tile, int lane, co
     R.v.pay.c1 = __builtin_nontemporal_load(reinterpret_cast<const u32*>(B.vcd + co + 256u));
     R.v.pay.c2 = __builtin_nontemporal_load(reinterpret_cast<const u32*>(B.vcd + co + 512u));
   }
+}
+// the lane's escape position from the tag words, and the 8 escape bytes from there on
+template <bool PAGED>
+__device__ __forceinline__ void load_tile_escapes(const Bases& B, int lane, const TagRegs& Tg, TileRegs& R) {
+  const int q = lane >> 4;
   // escape bytes per line of K (low half) and V (high half): one scan for both
   const u32 rb = (u32)esc_bytes(Tg.kfl) | ((u32)esc_bytes(Tg.vfl) << 16);
   const u32 excl = row_scan16(rb) - rb;
@@ -455,6 +465,11 @@ __device__ __forceinline__ void load_tile(const Bases& B, int tile, int lane, co
     R.k.e = load_u32x2_unaligned(B.kov + (u32)(Tg.kto + R.k.pos0));
     R.v.e = load_u32x2_unaligned(B.vov + (u32)(Tg.vto + R.v.pos0));
   }
+}
+template <bool PAGED>
+__device__ __forceinline__ void load_tile(const Bases& B, int tile, int lane, const TagRegs& Tg, TileRegs& R) {
+  load_tile_payload<PAGED>(B, tile, lane, Tg, R);
+  load_tile_escapes<PAGED>(B, lane, Tg, R);
 }
 
 // ---------------------------------------------------------------------------------------------------- one tile pair
@@ -670,12 +685,16 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
   else {
     // lengths known to the host (a Page) come as a kernel argument: the tile range, and with it the first payload loads, then depend on
     // nothing but the arguments
-    khs = A.k.head_start[ch]; vhs = A.v.head_start[ch];
-    TLh = (A.kt ? A.tl : A.k.head_start)[ch];      // no branch between the loads of this level
+    // These values are needed late (escape bytes, tail).  The index goes through a vector register the compiler knows nothing
+    // about, so that the loaded values stay in vector registers until readfirstlane fetches them where they are used; a value the
+    // compiler knows to be uniform is moved to a scalar register, and waited for, right where it is loaded.
+    int chv = ch;
+    asm volatile("" : "+v"(chv));
+    khs = A.k.head_start[chv]; vhs = A.v.head_start[chv];
+    TLh = (A.kt ? A.tl : A.k.head_start)[chv];      // no branch between the loads of this level
     if (HOST_LEN) S = A.S_all;
     else S = A.sl[ch];
     if (slot < 0) S = 0;
-    if (slot < 0 || !A.kt) TLh = 0;
   }
   if (tid < 256) tables_load_bases(Tr, tid, A.k.base3, A.k.base4, A.v.base3, A.v.base4, ch % A.NB);
 
@@ -695,8 +714,10 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
     __syncthreads();
   } else {
     const long rowb = (long)ch * A.S_pad, tileb = (long)ch * (A.S_pad / T);
-    B.ksm = A.k.sm + rowb * D; B.kcd = A.k.cd + rowb * CB; B.kfl = A.k.flags + rowb; B.kto = A.k.tile_off + tileb; B.kov = A.k.ovf + khs;
-    B.vsm = A.v.sm + rowb * D; B.vcd = A.v.cd + rowb * CB; B.vfl = A.v.flags + rowb; B.vto = A.v.tile_off + tileb; B.vov = A.v.ovf + vhs;
+    // (the escape streams start at head_start[ch], a loaded value: they are set where the first escape bytes are fetched, so that the
+    // loads issued until then do not wait for it)
+    B.ksm = A.k.sm + rowb * D; B.kcd = A.k.cd + rowb * CB; B.kfl = A.k.flags + rowb; B.kto = A.k.tile_off + tileb; B.kov = nullptr;
+    B.vsm = A.v.sm + rowb * D; B.vcd = A.v.cd + rowb * CB; B.vfl = A.v.flags + rowb; B.vto = A.v.tile_off + tileb; B.vov = nullptr;
     B.TS = 0;
   }
 
@@ -714,11 +735,14 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
   int iA = wave, iB = wave + NW;
   TileRegs R0, R1;
   TagRegs Tg, TgC0, TgC1;
-  if (iA < n_own) {          // start the first tile's loads before waiting for the block tables
-    load_tags<PAGED>(B, TT, TILE(iA), a, Tg);
-    TgC0 = Tg;
-    load_tile<PAGED>(B, TILE(iA), lane, Tg, R0);
-    load_tags<PAGED>(B, TT, TILE(min(iB, icl)), a, Tg);
+  const bool any_tile = iA < n_own;
+  // The wave's first tile: tag words and payload.  Without a branch where the addresses are always valid (a wave without tiles reads
+  // a tile it does not consume): behind a branch the compiler can no longer count the loads in flight and turns every later wait
+  // into a wait for all of them.  The escape bytes, which need the tag words and the stream start, follow after the block tables.
+  if (!PAGED || any_tile) {
+    const int tA = min(TILE(min(iA, icl)), max(ntiles - 1, 0));
+    load_tags<PAGED>(B, TT, tA, a, Tg);
+    load_tile_payload<PAGED>(B, tA, lane, Tg, R0);
   }
   if (tid == 0) next_tile = 2 * NW;
   // this launch's epoch of the fused merge: one more load of the start-up batch, its value is needed when the block is done
@@ -727,7 +751,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
   if (tid < 256) tables_store(L, Tr, tid, G);
   GAAC_STAMP(7);
   if (tid < GMAX) { M.m[NW][tid] = -INFINITY; M.l[NW][tid] = 0.f; }
-  __syncthreads();        // block tables are ready
+  lds_barrier();        // block tables are ready (a barrier that does not wait for the tile loads in flight)
   GAAC_STAMP(1);
   // Q as the B operand of the score product: lane (head a, quad q), product u covers group 4q+u in word order (e, e+4);
   // exponent-base words of the lane's units
@@ -742,7 +766,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
 
   // ---- the raw tail of the cache head: wave 0 of the last split's block, before it joins the tile hand-out
   if (!PAGED && A.kt && split == A.nsplit - 1 && wave == 0) {
-    const int TL = min(TLh, A.tcap);
+    const int TL = slot < 0 ? 0 : min(__builtin_amdgcn_readfirstlane(TLh), A.tcap);
     if (TL > 0) {
       // probabilities go through this wave's own merge slot: the other waves write theirs as soon as they run out of tiles
       float (*sc)[T] = reinterpret_cast<float (*)[T]>(&M.acc[0][0][0]);
@@ -751,8 +775,14 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
     }
   }
 
-  if (iA < n_own) {
+  if (!PAGED) { B.kov = A.k.ovf + __builtin_amdgcn_readfirstlane((int)khs); B.vov = A.v.ovf + __builtin_amdgcn_readfirstlane((int)vhs); }
+  if (any_tile) {
+    TgC0 = Tg;
+    load_tile_escapes<PAGED>(B, lane, Tg, R0);
+    load_tags<PAGED>(B, TT, TILE(min(iB, icl)), a, Tg);
     int vC = take_tile(&next_tile, n_own, lane);
+    // The loop is entered with the loads in flight in the same order as on its back edge (tile, then the next tile's tags), so the
+    // waits inside it stay waits for exactly the loads they need.
     while (true) {        // R0 = tile iA, Tg = tags of tile iB
       TgC1 = Tg;
       load_tile<PAGED>(B, TILE(min(iB, icl)), lane, Tg, R1);
