@@ -454,7 +454,7 @@ def bench_phases(a):
     dbg = torch.zeros(nblk * 16, dtype=torch.int64, device=dev)
     lib = _lib.load(); lib.gaac_set_phase_buffer.argtypes = [ctypes.c_void_p]; lib.gaac_set_phase_buffer.restype = None
     lib.gaac_set_phase_buffer(dbg.data_ptr())
-    f = lambda i: attn_launch(pages[i % len(pages)][0], pages[i % len(pages)][1], q2d, slots, n_q, N_KV, SL, S_CTX, D ** -0.5, nsplit, kt, vt, TL, 16, ws=ws)
+    f = lambda i: attn_launch(pages[i % len(pages)][0], pages[i % len(pages)][1], q2d, None if os.environ.get("PH_SALL") else slots, n_q, N_KV, SL, S_CTX, D ** -0.5, nsplit, kt, vt, TL, 16, ws=ws, S_all=S_CTX if os.environ.get("PH_SALL") else -1)
     for i in range(10): f(i)
     rows = []
     for i in range(20):

@@ -72,10 +72,10 @@ __device__ __forceinline__ u32 pack_bf16x2(float lo, float hi) {
 //     the whole record of this launch or an older one, never a torn one (naturally aligned 64-bit accesses are single-copy atomic),
 //     so no fence, flag or acknowledgement orders data against a separate signal.  Records are written with agent-scope stores
 //     (write-through) and read with agent-scope loads (they bypass the reader's L2): the blocks of a head sit on different XCDs.
-//   * The MERGERS are the head's last (up to eight) blocks in index order; each takes a share of the head's output (half a query head
+//   * The MERGERS are the head's last (up to sixteen) blocks in index order; each takes a share of the head's output (half a query head
 //     per wave), because one CU pulls records at only ~80 GB/s.  Once a merger has stored its own partial it loads the records of its
 //     share from all blocks of the head and re-reads those whose epoch is not yet the launch's.  Workgroups start in index order and
-//     a head's blocks are consecutive, so everything a merger waits for is running, done, or one of the at most seven later mergers
+//     a head's blocks are consecutive, so everything a merger waits for is running, done, or one of the at most fifteen later mergers
 //     of the same head, which get the next free CUs; blocks that are not mergers wait for nobody.  The wait is bounded all the same
 //     (MERGE_SPIN_LIMIT re-reads, then the rows are written as NaN), so that neither a damaged epoch word nor another start order
 //     can hang the GPU.
@@ -112,17 +112,34 @@ __device__ __forceinline__ void merge_half_head(const AttnArgs& A, long row, int
   const u64* rl = reinterpret_cast<const u64*>(A.pl) + row * nslot;
   const u64* ra = reinterpret_cast<const u64*>(A.pa) + row * nslot * D + d;
   float* fs = X.f[wave]; float* ls = X.l[wave];
-  constexpr int CH = 4;
+  constexpr int CH = 8;      // one round for up to 8 NW splits
   bool ok = true;
-  // all loads of the first round are issued before the first use: the wave's first CH accumulator rows, then m / l of slots 0..63
+  // all loads of the first round are issued before the first use: the wave's first CH accumulator rows ...
   u64 v[CH];
 #pragma unroll
   for (int k = 0; k < CH; ++k) { const int s = wave + NW * k; v[k] = s < nslot ? ll_load(ra + (long)s * D) : 0ull; }
-  float m = -INFINITY;
-  for (int s0 = 0; s0 < nslot; s0 += 64) {      // one pass for up to 64 splits
+  // ... then m / l of slots 0..63 (one slot per lane); everything is re-read together until it carries this launch's epoch
+  u64 mr = lane < nslot ? ll_load(rm + lane) : 0ull, lr = lane < nslot ? ll_load(rl + lane) : 0ull;
+  GAAC_MSTAMP(0, wall_clock64());
+  for (int spin = 0;; ++spin) {
+    bool stale = lane < nslot && (ll_stale(mr, epoch) || ll_stale(lr, epoch));
+#pragma unroll
+    for (int k = 0; k < CH; ++k) stale |= wave + NW * k < nslot && ll_stale(v[k], epoch);
+    if (__builtin_amdgcn_ballot_w64(stale) == 0) break;
+    if (spin >= MERGE_SPIN_LIMIT) { ok = false; break; }
+    __builtin_amdgcn_s_sleep(1);
+    if (lane < nslot && ll_stale(mr, epoch)) mr = ll_load(rm + lane);
+    if (lane < nslot && ll_stale(lr, epoch)) lr = ll_load(rl + lane);
+#pragma unroll
+    for (int k = 0; k < CH; ++k) { const int s = wave + NW * k; if (s < nslot && ll_stale(v[k], epoch)) v[k] = ll_load(ra + (long)s * D); }
+  }
+  GAAC_MSTAMP(1, wall_clock64());
+  float m = lane < nslot ? ll_value(mr) : -INFINITY;
+  if (lane < nslot) { fs[lane] = m; ls[lane] = ll_value(lr); }
+  for (int s0 = 64; ok && s0 < nslot; s0 += 64) {      // more than 64 splits: the other m / l records
     const int s = s0 + lane;
-    u64 mr = s < nslot ? ll_load(rm + s) : 0ull, lr = s < nslot ? ll_load(rl + s) : 0ull;
-    for (int spin = 0; ok && __builtin_amdgcn_ballot_w64(s < nslot && (ll_stale(mr, epoch) || ll_stale(lr, epoch))) != 0; ++spin) {
+    mr = s < nslot ? ll_load(rm + s) : 0ull; lr = s < nslot ? ll_load(rl + s) : 0ull;
+    for (int spin = 0; __builtin_amdgcn_ballot_w64(s < nslot && (ll_stale(mr, epoch) || ll_stale(lr, epoch))) != 0; ++spin) {
       if (spin >= MERGE_SPIN_LIMIT) { ok = false; break; }
       __builtin_amdgcn_s_sleep(1);
       if (s < nslot && ll_stale(mr, epoch)) mr = ll_load(rm + s);
@@ -130,31 +147,29 @@ __device__ __forceinline__ void merge_half_head(const AttnArgs& A, long row, int
     }
     if (s < nslot) { fs[s] = ll_value(mr); ls[s] = ll_value(lr); m = fmaxf(m, ll_value(mr)); }
   }
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  m = wave_max(m);
   float l = 0.f;
   for (int s = lane; s < nslot; s += 64) {      // each lane revisits the slots it wrote
     const float pmv = fs[s], f = pmv != -INFINITY ? __builtin_amdgcn_exp2f(pmv - m) : 0.f;
     fs[s] = f; l += ls[s] * f;
   }
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o, 64);
+  l = wave_sum(l);
   wave_lds_sync();
   float acc = 0.f;
   for (int s0 = wave; s0 < nslot; s0 += NW * CH) {
-    if (s0 != wave) {
+    if (s0 != wave) {      // more than CH * NW splits: the wave's further rows
 #pragma unroll
       for (int k = 0; k < CH; ++k) { const int s = s0 + NW * k; v[k] = s < nslot ? ll_load(ra + (long)s * D) : 0ull; }
-    }
-    for (int spin = 0; ok; ++spin) {
-      bool stale = false;
+      for (int spin = 0; ok; ++spin) {
+        bool stale = false;
 #pragma unroll
-      for (int k = 0; k < CH; ++k) stale |= s0 + NW * k < nslot && ll_stale(v[k], epoch);
-      if (__builtin_amdgcn_ballot_w64(stale) == 0) break;
-      if (spin >= MERGE_SPIN_LIMIT) { ok = false; break; }
-      __builtin_amdgcn_s_sleep(1);
+        for (int k = 0; k < CH; ++k) stale |= s0 + NW * k < nslot && ll_stale(v[k], epoch);
+        if (__builtin_amdgcn_ballot_w64(stale) == 0) break;
+        if (spin >= MERGE_SPIN_LIMIT) { ok = false; break; }
+        __builtin_amdgcn_s_sleep(1);
 #pragma unroll
-      for (int k = 0; k < CH; ++k) { const int s = s0 + NW * k; if (s < nslot && ll_stale(v[k], epoch)) v[k] = ll_load(ra + (long)s * D); }
+        for (int k = 0; k < CH; ++k) { const int s = s0 + NW * k; if (s < nslot && ll_stale(v[k], epoch)) v[k] = ll_load(ra + (long)s * D); }
+      }
     }
 #pragma unroll
     for (int k = 0; k < CH; ++k) {
@@ -162,21 +177,24 @@ __device__ __forceinline__ void merge_half_head(const AttnArgs& A, long row, int
       if (s < nslot) { const float f = fs[s]; acc += f != 0.f ? ll_value(v[k]) * f : 0.f; }      // an empty partial's accumulator may hold anything
     }
   }
+  GAAC_MSTAMP(2, wall_clock64());
   X.part[wave][lane] = acc;
   if (lane == 0) X.ok[wave] = ok;
   lds_barrier();
+  GAAC_MSTAMP(3, wall_clock64());
   if (wave == 0) {
 #pragma unroll
     for (int w = 1; w < NW; ++w) { acc += X.part[w][lane]; ok = ok && X.ok[w]; }
     const float o = ok ? (l > 0.f ? acc / l : 0.f) : __builtin_nanf("");
     A.out[row * D + d] = __builtin_bit_cast(u16, (__bf16)o);
   }
+  GAAC_MSTAMP(4, wall_clock64());
   lds_barrier();      // part is free for the block's next item
 }
 // The merge of a head is shared by its last `mergers` blocks in index order (merge_ranks): the block of rank j takes the half heads
 // j, j + mergers, ..., so that no single CU has to pull all the records.  Called by all threads of a merging block after its own
 // partial has been stored and every thread is done with the LDS that X aliases.
-__device__ __forceinline__ int merge_ranks(int G, int nslot) { return min(min(8, 2 * G), nslot); }
+__device__ __forceinline__ int merge_ranks(int G, int nslot) { return min(min(16, 2 * G), nslot); }
 template <int NW>
 __device__ __forceinline__ void merge_heads(const AttnArgs& A, long qh0, int G, u32 epoch, int rank, int mergers, int tid, MergeScratch<NW>& X) {
   const int wave = tid >> 6, lane = tid & 63;

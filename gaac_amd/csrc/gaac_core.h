@@ -88,6 +88,16 @@ __device__ __forceinline__ float quad_rows_sum(float v) {
   return __uint_as_float(s[0]) + __uint_as_float(s[1]);
 }
 
+// all-reduce over the 64 lanes of the wave without LDS traffic: four DPP steps inside each 16-lane row, then across the rows
+#define GAAC_ROW16_REDUCE(v, OP)                                                   \
+  v = OP(v, __uint_as_float((u32)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), 0xB1, 0xF, 0xF, true)));  /* quad_perm [1,0,3,2] */ \
+  v = OP(v, __uint_as_float((u32)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), 0x4E, 0xF, 0xF, true)));  /* quad_perm [2,3,0,1] */ \
+  v = OP(v, __uint_as_float((u32)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), 0x141, 0xF, 0xF, true))); /* row_half_mirror */      \
+  v = OP(v, __uint_as_float((u32)__builtin_amdgcn_update_dpp(0, (int)__float_as_uint(v), 0x140, 0xF, 0xF, true)))  /* row_mirror */
+__device__ __forceinline__ float gaac_addf(float a, float b) { return a + b; }
+__device__ __forceinline__ float wave_max(float v) { GAAC_ROW16_REDUCE(v, fmaxf); return quad_rows_max(v); }
+__device__ __forceinline__ float wave_sum(float v) { GAAC_ROW16_REDUCE(v, gaac_addf); return quad_rows_sum(v); }
+
 // ---- exponent-base words ------------------------------------------------------------------------------------------
 // Word p of a group pairs elements p (low half) and p+4 (high half): base << 7 | base' << 23 sits on the exponent fields.
 template <int KIND>

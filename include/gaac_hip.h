@@ -76,7 +76,7 @@ int gaac_attn_split(
 int gaac_attn_combine(const float* pm, const float* pl, const float* pa, void* out, int n_rows, int nslot, void* stream);
 
 /* gaac_attn_launch as ONE kernel: the merge of the NSLOT partials (gaac_combine, kernel.py:281-294) is done inside the split kernel
- * by the last (up to eight) blocks of each (batch row, kv head) in index order, each taking a share of the head's output, without
+ * by the last (up to sixteen) blocks of each (batch row, kv head) in index order, each taking a share of the head's output, without
  * atomics.  *epoch holds the epoch of the last merged launch; this launch's epoch is that + 1.  Partials travel as 64-bit records
  * (fp32 bits | epoch << 32) written and read with single 64-bit accesses, so a merging block recognises the records of this launch
  * without waiting for an acknowledgement; it re-reads records that have not arrived yet (bounded; rows are written as NaN if they
