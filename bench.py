@@ -23,7 +23,8 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the attention kernel on the default workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by the
 # library's plain 64 MiB copy kernel (factors 1.99937 read, 1.0 write); the profiler runs are separate from a timing run, so the
 # figure is carried here and reported only for the configuration it was measured on.
-MEASURED_TRAFFIC = {"nsplit": 32, "bytes": 194632199}
+MEASURED_TRAFFIC = {"nsplit": 32, "bytes": 194632199,
+                    "source": "constant in bench.py, not measured by this run: profiles/k_attn_split_config1_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)"}
 
 
 def make_kv(seed: int, H: int, S: int, lo: float = -4.0, hi: float = 4.0) -> torch.Tensor:
@@ -54,24 +55,47 @@ def clone_store(page):
     return c
 
 
-def cpu_baseline(k16: np.ndarray, v16: np.ndarray, q16: np.ndarray, b3k, b4k, b3v, b4v, scale: float, heads: int, reps: int = 4) -> dict:
-    """The CPU oracle's decompress + fp32 softmax attention on `heads` kv heads of the same workload (bounded sample),
-    timed on this box's host cores; pages are encoded beforehand (not timed)."""
+_CPU_PAGES = None      # per-head oracle pages of the CPU baseline, inherited by its forked workers
+
+
+def _cpu_head_pass(h: int):
+    """One kv head of the CPU baseline: oracle decode of its K and V pages + fp32 softmax attention of its G query heads."""
     from oracle import gaac_oracle as O
     from threadpoolctl import threadpool_limits
-    kp = O.encode(k16[:heads], "k", b3k[:heads], b4k[:heads], heads)
-    vp = O.encode(v16[:heads], "v", b3v[:heads], b4v[:heads], heads)
+    kp, vp, q16, scale = _CPU_PAGES[h]
     with threadpool_limits(limits=1):
+        kd, vd = O.decode(kp), O.decode(vp)
+        out = O.ref_attention(q16, kd.transpose(1, 0, 2), vd.transpose(1, 0, 2), scale)
+    return kd, vd, out
+
+
+def cpu_baseline(k16: np.ndarray, v16: np.ndarray, q16: np.ndarray, b3k, b4k, b3v, b4v, scale: float, heads: int, reps: int = 3) -> dict:
+    """The CPU oracle's decompress + fp32 softmax attention on `heads` kv heads of the same workload (bounded sample), timed on this
+    box's host cores: once on one thread, once with one worker process per kv head.  Pages are encoded beforehand (not timed)."""
+    global _CPU_PAGES
+    import multiprocessing as mp
+    from oracle import gaac_oracle as O
+    _CPU_PAGES = [(O.encode(k16[h:h + 1], "k", b3k[h:h + 1], b4k[h:h + 1], 1), O.encode(v16[h:h + 1], "v", b3v[h:h + 1], b4v[h:h + 1], 1),
+                   q16[h * G:(h + 1) * G], scale) for h in range(heads)]
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        res = [_cpu_head_pass(h) for h in range(heads)]
+    dt1 = (time.perf_counter() - t0) / reps
+    for h, (kd, vd, out) in enumerate(res):
+        assert np.array_equal(kd[0], k16[h]) and np.array_equal(vd[0], v16[h]) and np.isfinite(out).all()
+    workers = max(1, min(heads, len(os.sched_getaffinity(0)), 16))
+    with mp.get_context("fork").Pool(workers) as pool:
+        pool.map(_cpu_head_pass, range(heads))      # warm-up: workers started, pages touched
         t0 = time.perf_counter()
-        for _ in range(reps):
-            kd, vd = O.decode(kp), O.decode(vp)
-            out = O.ref_attention(q16[:heads * G], kd.transpose(1, 0, 2), vd.transpose(1, 0, 2), scale)
-        dt = (time.perf_counter() - t0) / reps
-    assert np.array_equal(kd, k16[:heads]) and np.array_equal(vd, v16[:heads]) and np.isfinite(out).all()
-    us_layer = dt * 1e6 * (N_KV / heads)
-    return {"value": us_layer, "unit": "us/layer", "cores": 1, "kind": "port",
-            "sample": f"{heads} of {N_KV} kv heads x {k16.shape[1]} tokens (K and V): numpy oracle decode + fp32 softmax attention, "
-                      f"mean of {reps} passes of {dt:.1f} s, scaled x{N_KV / heads:g}; host has {os.cpu_count()} cpus, 1 thread used"}
+        for _ in range(reps): pool.map(_cpu_head_pass, range(heads))
+        dtn = (time.perf_counter() - t0) / reps
+    _CPU_PAGES = None
+    scale_up = N_KV / heads
+    return {"value": dtn * 1e6 * scale_up, "unit": "us/layer", "cores": workers, "kind": "port",
+            "one_thread_us_per_layer": dt1 * 1e6 * scale_up,
+            "sample": f"{heads} of {N_KV} kv heads x {k16.shape[1]} tokens (K and V): numpy oracle decode + fp32 softmax attention per kv head; "
+                      f"mean of {reps} passes: {dt1:.2f} s on 1 thread, {dtn:.2f} s with {workers} worker processes (one kv head each), scaled x{scale_up:g}; "
+                      f"host offers {len(os.sched_getaffinity(0))} cpus"}
 
 
 def main():
@@ -82,6 +106,7 @@ def main():
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="also run the library's plain 64 MiB copy kernel 10 times (the known-size kernel for scaling FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--cpu-heads", type=int, default=8, help="kv heads in the CPU baseline sample (0 = skip)")
+    ap.add_argument("--kernel-only", action="store_true", help="decode64k: time the compressed kernel only (no baselines): the run to put under rocprofv3")
     ap.add_argument("--workload", default="decode64k", choices=["decode64k", "decode64k_g6", "codec", "paged", "serve", "phases"],
                     help="decode64k = the headline (config 1); decode64k_g6 = config 2 (24 q / 4 kv heads, V sigma in 2^[-2,2]); "
                          "codec = config 0 round trip; paged = config 3 serving step; serve = config 4 end-to-end decode; "
@@ -128,7 +153,8 @@ def main():
 
     def step(i, phase="fused"):
         K, V = pages[i % len(pages)]
-        return attn_launch(K, V, q2d, None, n_q, N_KV, SL, S_pad, scale, nsplit, kt, vt, TL, 16, ws=ws, phase=phase)      # rows in order, as gaac.kernel.attention
+        # rows in order and lengths known to the host, as gaac.kernel.attention passes them for two Pages
+        return attn_launch(K, V, q2d, None, n_q, N_KV, SL, S_pad, scale, nsplit, kt, vt, TL, 16, ws=ws, phase=phase, S_all=S_CTX)
 
     if a.traffic_calibration:
         from gaac_amd import _lib
@@ -144,10 +170,18 @@ def main():
     assert torch.equal(kdec[:, :S_CTX].to(torch.bfloat16).view(torch.int16), kd[:, :S_CTX].view(torch.int16)), "round trip is not bit-exact"
     sc = torch.einsum("hgd,hsd->hgs", q2d.float().view(H, G, D), kdec) * scale
     ref = torch.einsum("hgs,hsd->hgd", torch.softmax(sc, -1), vdec).reshape(B * n_q, D)
-    err_max, err_mean = (out - ref).abs().max().item(), (out - ref).abs().mean().item()
+    err_max, err_mean, ref_max = (out - ref).abs().max().item(), (out - ref).abs().mean().item(), ref.abs().max().item()
     del kdec, vdec, sc
+    # the bar of the headline: max-abs 1e-2 and mean-abs 1e-3 against decompress + fp32 softmax attention; for more batch rows (other
+    # sequences, other magnitudes) the reference's own relative tolerance (tests/test_kernel.py:19)
+    if B == 1: assert err_max <= 1e-2 and err_mean <= 1e-3, f"attention error max {err_max:.3e} mean {err_mean:.3e} (max |ref| {ref_max:.3f})"
+    else: assert err_max <= 2e-2 * ref_max + 1e-3, f"attention error max {err_max:.3e} (max |ref| {ref_max:.3f})"
 
-    # ---- timed region: K steps captured in one HIP graph (no host launch gaps), replayed once between synchronizes
+    # ---- timed region: the K steps are captured in one HIP graph (no host launch gaps), as many times over as it takes to reach about
+    # 1000 launches per graph (starting a graph costs ~40 us on the GPU's timeline, which a short graph would add to every step), and the
+    # graph is replayed back to back until at least ~50 ms have been timed, so that the figure does not depend on K.  Wall clock between
+    # synchronizes gives `value`; HIP events on the launch stream around the same replays give the kernel's mean duration (launch to
+    # launch, idle gaps between dependent launches included), from which the roofline figure is taken.
     for i in range(a.warmup): step(i)
     torch.cuda.synchronize()
     side = torch.cuda.Stream()
@@ -155,29 +189,55 @@ def main():
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.stream(side):
         step(0); torch.cuda.synchronize()
+        per_graph = a.steps * max(1, -(-1000 // a.steps))
         with torch.cuda.graph(graph, stream=side):
-            for i in range(a.steps): step(i)
+            for i in range(per_graph): step(i)
     torch.cuda.synchronize()
     graph.replay(); torch.cuda.synchronize()          # untimed replay (graph upload)
+    t0 = time.perf_counter(); graph.replay(); torch.cuda.synchronize()
+    est = time.perf_counter() - t0
+    replays = max(1, min(2000, int(math.ceil(0.05 / max(est, 1e-6)))))
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
-    graph.replay()
+    with torch.cuda.stream(side):
+        e0.record(side)
+        for _ in range(replays): graph.replay()
+        e1.record(side)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    us_step = dt * 1e6 / a.steps
+    n_timed = per_graph * replays
+    us_step = dt * 1e6 / n_timed
+    split_us_mean = e0.elapsed_time(e1) * 1e3 / n_timed
 
-    # ---- duration of the attention kernel itself: HIP events on the launch stream around batches of back-to-back launches
-    # (one event pair per launch would add the event's own ~3 us to every sample)
-    BATCH = 20
-    nb = min(max(5, a.steps // BATCH), 30)
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(nb)]
-    for b_, (e0, e1) in enumerate(evs):
-        e0.record()
-        for i in range(BATCH): step(b_ * BATCH + i)
-        e1.record()
-    torch.cuda.synchronize()
-    ts = sorted(e0.elapsed_time(e1) * 1e3 / BATCH for e0, e1 in evs)
-    split_us_mean, split_us_med = sum(ts) / len(ts), ts[len(ts) // 2]
-
+    # ---- the floor the load pattern sets: the library's read probe (the kernel's loads over the same pages, no arithmetic), timed the same way
+    def time_graph(fn):
+        g = torch.cuda.CUDAGraph()
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            fn(0); torch.cuda.synchronize()
+            with torch.cuda.graph(g, stream=side):
+                for i in range(per_graph): fn(i)
+        torch.cuda.synchronize(); g.replay(); torch.cuda.synchronize()
+        t0_ = time.perf_counter()
+        with torch.cuda.stream(side):
+            for _ in range(replays): g.replay()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0_) * 1e6 / n_timed
+    from gaac_amd import _lib
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    def probe(i, meta):
+        K, V = pages[i % len(pages)]
+        P = _lib.ptr
+        _lib.call("gaac_read_probe", P(K.sm), P(K.codes), P(K.flags), P(K.tile_off), P(K.ovf), P(K.ovf_head_start),
+                  P(V.sm), P(V.codes), P(V.flags), P(V.tile_off), P(V.ovf), P(V.ovf_head_start), H, S_CTX, S_pad, nsplit, meta, P(sink), _lib.stream())
+    probe_us = {"payload_only_us": round(time_graph(lambda i: probe(i, 0)), 2), "with_tags_and_escapes_us": round(time_graph(lambda i: probe(i, 1)), 2),
+                "what": "gaac_read_probe: the attention kernel's loads over the same pages without its arithmetic, same blocks and splits, timed like the kernel"}
+    if a.kernel_only:
+        print(json.dumps({"workload": f"config {1 if G == 4 else 2} kernel only", "value": round(us_step, 3), "unit": "us/layer", "steps_timed": n_timed, "nsplit": nsplit,
+                          "kernel_us_mean": round(split_us_mean, 3), "algorithmic_bytes": alg_bytes, "frac_of_8TBps": round(alg_bytes / split_us_mean / 1e3 / HBM_PEAK_GBS, 4),
+                          "read_probe": probe_us, "check": {"max_abs": err_max, "mean_abs": err_mean, "max_abs_ref": ref_max}}))
+        return
     # ---- uncompressed BF16 decode attention on the same GPU over the same tokens (compressed part + tail, contiguous), rotating copies:
     # (a) the library's own baseline kernel = this kernel's structure without the decoder, best of a few split counts;
     # (b) torch's scaled_dot_product_attention, for reference only
@@ -187,19 +247,21 @@ def main():
     ref_b = bf16_attention(qb, kb[0], vb[0], scale).float().view(B * n_q, D)
     assert (ref_b - ref).abs().max().item() <= 2e-2 * ref.abs().max().item() + 1e-3, "baseline kernel is off"      # the reference's tolerance
     bf16_us, bf16_ns = None, None
-    for ns in sorted({max(1, x // B) for x in (64, 96, 128, 192)}):
+    for ns in sorted({max(1, x // B) for x in (32, 64, 96, 128)}):      # 32: eight-wave blocks like the compressed kernel; more: four-wave blocks
         wsb = AttnWorkspace(B * n_q, ns, torch.bfloat16, dev)
         outb = torch.empty(B * n_q, D, dtype=torch.bfloat16, device=dev)
         for i in range(10): bf16_attention(qb, kb[i % a.copies], vb[i % a.copies], scale, ns, wsb, out=outb)
-        n_b = min(max(60, a.steps // 2), 300)
-        gb = torch.cuda.CUDAGraph()                      # timed like the compressed kernel: one graph of launches, wall clock
+        gb = torch.cuda.CUDAGraph()                      # timed like the compressed kernel: a graph of the K steps replayed back to back
         torch.cuda.synchronize()
         with torch.cuda.stream(side):
             with torch.cuda.graph(gb, stream=side):
-                for i in range(n_b): bf16_attention(qb, kb[i % a.copies], vb[i % a.copies], scale, ns, wsb, out=outb)
+                for i in range(per_graph): bf16_attention(qb, kb[i % a.copies], vb[i % a.copies], scale, ns, wsb, out=outb)
         torch.cuda.synchronize(); gb.replay(); torch.cuda.synchronize()
-        t0b = time.perf_counter(); gb.replay(); torch.cuda.synchronize()
-        t = (time.perf_counter() - t0b) * 1e6 / n_b
+        t0b = time.perf_counter()
+        with torch.cuda.stream(side):
+            for _ in range(replays): gb.replay()
+        torch.cuda.synchronize()
+        t = (time.perf_counter() - t0b) * 1e6 / n_timed
         del gb
         if bf16_us is None or t < bf16_us: bf16_us, bf16_ns = t, ns
     q4 = qd.view(B, n_q, 1, D)
@@ -218,18 +280,23 @@ def main():
         "n_gpus": 1, "steps": a.steps, "warmup": a.warmup, "ms_per_step": round(us_step / 1e3, 6), "higher_is_better": False,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"config {1 if G == 4 else 2}: fused decode attention, batch {B}, {n_q} q heads / {N_KV} kv heads, d=128, 65536 compressed tokens + 7-token bf16 tail",
-                   "nsplit": nsplit, "kv_copies_rotated": len(pages), "timing": "one HIP graph of all steps, wall clock between synchronizes"},
+                   "nsplit": nsplit, "kv_copies_rotated": len(pages),
+                   "timing": f"one HIP graph holding the {a.steps} steps {per_graph // a.steps} times over, replayed {replays} times back to back "
+                             f"({n_timed} steps timed), wall clock between synchronizes"},
         "effective_GBps": round(alg_bytes / us_step / 1e3, 1), "algorithmic_bytes": alg_bytes, "bf16_bytes": bf16_bytes,
         "compression_ratio_k": round(kp.ratio, 4), "compression_ratio_v": round(vp.ratio, 4),
         "tier_shares_k": [round(s3k, 4), round(s4k, 4), round(srk, 5)], "tier_shares_v": [round(s3v, 4), round(s4v, 4), round(srv, 5)],
-        "check": {"vs": "fp32 softmax attention (torch, device) over HIP-decoded KV", "max_abs": err_max, "mean_abs": err_mean, "roundtrip_bit_exact": True},
-        "bf16_baseline": {"kernel": "k_bf16_attn_split (same structure, no decoder)", "us": round(bf16_us, 2), "nsplit": bf16_ns,
+        "check": {"vs": "fp32 softmax attention (torch, device) over HIP-decoded KV", "max_abs": err_max, "mean_abs": err_mean, "max_abs_ref": ref_max,
+                  "asserted": "max_abs <= 1e-2 and mean_abs <= 1e-3" if B == 1 else "max_abs <= 2e-2 * max_abs_ref + 1e-3", "roundtrip_bit_exact": True},
+        "bf16_baseline": {"kernel": "k_bf16_attn_split (same structure, block shapes and merge, no decoder; best of 4 split counts)", "us": round(bf16_us, 2), "nsplit": bf16_ns,
                           "GBps": round(bf16_bytes / bf16_us / 1e3, 1), "speedup_of_compressed": round(bf16_us / us_step, 3),
                           "torch_sdpa_us": round(sdpa_us, 1)},
         "roofline": {"bound": "hbm", "achieved": round(alg_bytes / split_us_mean / 1e3, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(alg_bytes / split_us_mean / 1e3 / HBM_PEAK_GBS, 4),
                      "traffic": MEASURED_TRAFFIC["bytes"] if nsplit == MEASURED_TRAFFIC["nsplit"] and a.workload == "decode64k" and B == 1 else None,
-                     "kernel": "k_attn_split (split pass + tail + fused merge)", "kernel_us_mean": round(split_us_mean, 2), "kernel_us_median": round(split_us_med, 2)},
+                     "traffic_source": MEASURED_TRAFFIC["source"],
+                     "kernel": "k_attn_split (split pass + tail + fused merge)", "kernel_us_mean": round(split_us_mean, 2),
+                     "kernel_us_from": "HIP events on the launch stream around the timed graph replays / steps timed", "read_probe": probe_us},
     }
     if a.cpu_heads > 0 and B == 1:
         b = lambda t: t.cpu().numpy()

@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libgaac_hip.so")
 LIB_TIMING = os.path.join(HERE, "libgaac_hip_timing.so")      # same sources with -DGAAC_PHASE_TIMING (per-block phase time stamps)
-SOURCES = ["codec.hip", "attn.hip", "cache.hip", "paged.hip"]
+SOURCES = ["codec.hip", "attn.hip", "cache.hip", "paged.hip", "probe.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", 
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",      # never emit packed-FP32 VALU ops
          # atomics here are issued by one chosen lane (tile counter in LDS, merge ticket): skip the compiler's wave-wide aggregation code

@@ -1003,9 +1003,12 @@ __device__ __forceinline__ void consume_raw_tile(const RawTile& R, WaveState& st
   }
 }
 
-struct Bf16Lds { u32x4 qw[GMAX][NG]; float m[4][GMAX], l[4][GMAX]; float acc[5][GMAX][D]; };      // acc: also the mergers' scratch
-__global__ void __launch_bounds__(256, 2) k_bf16_attn_split(const AttnArgs A) {
-  __shared__ Bf16Lds L;
+// NW as in k_attn_split: eight-wave blocks (one per CU) for launches of up to 256 blocks, else four-wave blocks (two per CU)
+template <int NW> struct Bf16Lds { u32x4 qw[GMAX][NG]; float m[NW][GMAX], l[NW][GMAX]; float acc[NW + 1][GMAX][D]; };      // acc: also the mergers' scratch
+template <int NW>
+__global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_bf16_attn_split(const AttnArgs A) {
+  constexpr int NT = 64 * NW;
+  __shared__ Bf16Lds<NW> L;
   const int bh = (int)blockIdx.x / A.nsplit, split = (int)blockIdx.x % A.nsplit, tid = threadIdx.x;      // a head's blocks are consecutive
   const int b = bh / A.n_kv, kvh = bh % A.n_kv, G = A.G;
   const long qh0 = (long)b * A.n_q + (long)kvh * G;
@@ -1018,13 +1021,13 @@ __global__ void __launch_bounds__(256, 2) k_bf16_attn_split(const AttnArgs A) {
   __shared__ int next_tile;
   const bool part_here = (S % T) != 0 && thi == ntiles && thi > tlo;
   const int thd = thi - (part_here ? 1 : 0), tcl = max(thd - 1, tlo);
-  int tA = tlo + wave, tB = tA + 4;
+  int tA = tlo + wave, tB = tA + NW;
   RawTile R0, R1;
   if (tA < thd) load_raw_tile(kh, vh, tA, S, a, q, R0);
-  if (tid == 0) next_tile = tlo + 8;
+  if (tid == 0) next_tile = tlo + 2 * NW;
   const u32 epoch = load_epoch(A, bh);
   // Q as the B operand: lane (head a, quad q), product j covers channels 32 j + 8 q .. + 8 (rows >= G are zero)
-  for (int i = tid; i < GMAX * NG; i += 256) {
+  for (int i = tid; i < GMAX * NG; i += NT) {
     const int h = i >> 4, c = i & 15;
     L.qw[h][c] = h < G ? *reinterpret_cast<const u32x4*>(A.q + (qh0 + h) * D + 8 * c) : u32x4{0u, 0u, 0u, 0u};
   }
@@ -1066,13 +1069,13 @@ __global__ void __launch_bounds__(256, 2) k_bf16_attn_split(const AttnArgs A) {
   __syncthreads();
   const int mergers = merge_ranks(G, A.nslot), rank = split - (A.nsplit - mergers);
   const int d = tid & 127;
-  for (int g = tid >> 7; g < G; g += 2) {
+  for (int g = tid >> 7; g < G; g += NT / 128) {
     float M = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) M = fmaxf(M, L.m[w][g]);
+    for (int w = 0; w < NW; ++w) M = fmaxf(M, L.m[w][g]);
     float Lc = 0.f, Ac = 0.f;
 #pragma unroll
-    for (int w = 0; w < 4; ++w) {
+    for (int w = 0; w < NW; ++w) {
       const float f = L.m[w][g] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(L.m[w][g] - M);
       Lc += L.l[w][g] * f; Ac += L.acc[w][g][d] * f;
     }
@@ -1085,7 +1088,7 @@ __global__ void __launch_bounds__(256, 2) k_bf16_attn_split(const AttnArgs A) {
   }
   if (rank >= 0 && A.nslot > 1) {
     lds_barrier();
-    merge_heads<4>(A, qh0, G, epoch, rank, mergers, tid, *reinterpret_cast<MergeScratch<4>*>(&L.acc[0][0][0]));
+    merge_heads<NW>(A, qh0, G, epoch, rank, mergers, tid, *reinterpret_cast<MergeScratch<NW>*>(&L.acc[0][0][0]));
   }
 }
 
@@ -1215,6 +1218,7 @@ extern "C" int gaac_bf16_attn(const void* k, const void* v, int S, const int* se
   A.n_kv = n_kv; A.n_q = n_q; A.G = n_q / n_kv; A.NB = 1;
   A.kt = (const u16*)k; A.vt = (const u16*)v; A.tcap = S; A.sl = seq_lens;
   A.epochs = epoch; A.out = (u16*)out;
-  hipLaunchKernelGGL(k_bf16_attn_split, dim3(B * n_kv * nsplit), dim3(256), 0, (hipStream_t)stream, A);
+  if ((long)B * n_kv * nsplit <= 256) hipLaunchKernelGGL(k_bf16_attn_split<8>, dim3(B * n_kv * nsplit), dim3(512), 0, (hipStream_t)stream, A);
+  else hipLaunchKernelGGL(k_bf16_attn_split<4>, dim3(B * n_kv * nsplit), dim3(256), 0, (hipStream_t)stream, A);
   return launch_status("gaac_bf16_attn");
 }

@@ -1,0 +1,75 @@
+// Measurement aid: the memory side of the fused decode-attention kernel without its arithmetic.  One block per (cache head, split), eight
+// waves, every wave fetches the tiles wave, wave + 8, ... of the block's contiguous range one tile ahead of the tile it "consumes" (an
+// xor over the loaded registers), with the attention kernel's own loads: per tile and kind two 16-byte and three 4-byte loads per lane
+// (non-temporal), and, on request, the tile's tag words, its offset in the escape stream and eight escape bytes per lane.  What this
+// kernel needs for a page is what the load pattern itself costs on the part: the floor under k_attn_split for that page.
+#include "gaac_tile.h"
+#include "gaac_capi.h"
+#include "../../include/gaac_hip.h"
+
+namespace gaac {
+
+struct ProbeView { const uint8_t* sm; const uint8_t* cd; const int* flags; const int* tile_off; const uint8_t* ovf; const int* head_start; };
+struct ProbeRegs { Payload k, v; u32 kf, vf, kto, vto; u32x2 ke, ve; };
+
+template <bool META>
+__device__ __forceinline__ void probe_load(const ProbeView& K, const ProbeView& V, long rowb, long tileb, long khs, long vhs, int tile, int lane, ProbeRegs& R) {
+  const u32 so = (u32)tile * TILE_SM, co = (u32)tile * TILE_CD;
+  load_payload(K.sm + rowb * D + so, K.cd + rowb * CB + co, lane, R.k);
+  load_payload(V.sm + rowb * D + so, V.cd + rowb * CB + co, lane, R.v);
+  if (META) {
+    const int a = lane & 15;
+    R.kf = (u32)__builtin_nontemporal_load(K.flags + rowb + tile * T + a); R.vf = (u32)__builtin_nontemporal_load(V.flags + rowb + tile * T + a);
+    R.kto = (u32)K.tile_off[tileb + tile]; R.vto = (u32)V.tile_off[tileb + tile];
+  }
+}
+__device__ __forceinline__ u32 probe_fold(const ProbeRegs& R) {
+  return R.k.s0[0] ^ R.k.s0[3] ^ R.k.s1[1] ^ R.k.s1[2] ^ R.k.c0 ^ R.k.c1 ^ R.k.c2 ^ R.v.s0[0] ^ R.v.s0[3] ^ R.v.s1[1] ^ R.v.s1[2] ^ R.v.c0 ^ R.v.c1 ^ R.v.c2;
+}
+// META: also the tag words, tile offsets and escape bytes (the escape loads wait for the tag words of their tile, as in the attention
+// kernel: a lane's escape position is a prefix over the tag words)
+template <bool META>
+__global__ void __launch_bounds__(512, 1) k_read_probe(ProbeView K, ProbeView V, int S_pad, int ntiles, int nsplit, u32* __restrict__ sink) {
+  constexpr int NW = 8;
+  const int ch = (int)blockIdx.x / nsplit, split = (int)blockIdx.x % nsplit, wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int chunk = (ntiles + nsplit - 1) / nsplit, tlo = min(split * chunk, ntiles), n_own = min(tlo + chunk, ntiles) - tlo;
+  const long rowb = (long)ch * S_pad, tileb = (long)ch * (S_pad / T);
+  const long khs = META ? K.head_start[ch] : 0, vhs = META ? V.head_start[ch] : 0;
+  if (wave >= n_own) return;
+  const int last = tlo + n_own - 1;
+  ProbeRegs R0, R1;
+  u32 acc = 0u;
+  auto escapes = [&](ProbeRegs& R) {
+    if (META) {
+      const u32 rb = (u32)esc_bytes(R.kf) | ((u32)esc_bytes(R.vf) << 16), excl = row_scan16(rb) - rb;
+      R.ke = load_u32x2_unaligned(K.ovf + khs + R.kto + (excl & 0xFFFFu) + (u32)esc_prefix(R.kf, 8 * (lane >> 4)));
+      R.ve = load_u32x2_unaligned(V.ovf + vhs + R.vto + (excl >> 16) + (u32)esc_prefix(R.vf, 8 * (lane >> 4)));
+    }
+  };
+  auto fold = [&](const ProbeRegs& R) { acc ^= probe_fold(R); if (META) acc ^= R.ke[0] ^ R.ke[1] ^ R.ve[0] ^ R.ve[1]; };
+  probe_load<META>(K, V, rowb, tileb, khs, vhs, tlo + wave, lane, R0); escapes(R0);
+  for (int i = wave; i < n_own; i += 2 * NW) {
+    probe_load<META>(K, V, rowb, tileb, khs, vhs, min(tlo + i + NW, last), lane, R1); escapes(R1);
+    fold(R0);
+    if (i + NW >= n_own) break;
+    probe_load<META>(K, V, rowb, tileb, khs, vhs, min(tlo + i + 2 * NW, last), lane, R0); escapes(R0);
+    fold(R1);
+  }
+  if (acc == 0x9E3779B9u) sink[0] = acc;      // keeps the loads alive; practically never written
+}
+
+}  // namespace gaac
+
+using namespace gaac;
+
+extern "C" int gaac_read_probe(
+    const uint8_t* smk, const uint8_t* ck, const int* fk, const int* tok, const uint8_t* ovk, const int* ohsk,
+    const uint8_t* smv, const uint8_t* cv, const int* fv, const int* tov, const uint8_t* ovv, const int* ohsv,
+    int H, int S, int S_pad, int nsplit, int with_meta, unsigned int* sink, void* stream) {
+  GAAC_REQUIRE(smk && ck && fk && tok && ovk && ohsk && smv && cv && fv && tov && ovv && ohsv && sink, "gaac_read_probe: null pointer");
+  GAAC_REQUIRE(H > 0 && S > 0 && S % T == 0 && S <= S_pad && S_pad % T == 0 && nsplit >= 1, "gaac_read_probe: bad sizes H=%d S=%d S_pad=%d nsplit=%d", H, S, S_pad, nsplit);
+  const ProbeView K{smk, ck, fk, tok, ovk, ohsk}, V{smv, cv, fv, tov, ovv, ohsv};
+  if (with_meta) hipLaunchKernelGGL(k_read_probe<true>, dim3(H * nsplit), dim3(512), 0, (hipStream_t)stream, K, V, S_pad, S / T, nsplit, sink);
+  else hipLaunchKernelGGL(k_read_probe<false>, dim3(H * nsplit), dim3(512), 0, (hipStream_t)stream, K, V, S_pad, S / T, nsplit, sink);
+  return launch_status("gaac_read_probe");
+}

@@ -148,6 +148,16 @@ int gaac_bf16_attn(const void* k, const void* v, int S, const int* seq_lens, lon
  * the known-size kernel that HBM traffic counters (FETCH_SIZE / WRITE_SIZE) are scaled against. */
 int gaac_stream_copy(const void* src, void* dst, long nbytes, void* stream);
 
+/* Measurement aid with no counterpart in the reference: the memory side of gaac_attn_fused without its arithmetic.  One eight-wave
+ * block per (cache head, split) streams the K and V page tensors (the first twelve arguments of gaac_attn_fused, without the bases) of
+ * H heads x S tokens (S a multiple of 16) with the attention kernel's own loads, one tile ahead; with_meta != 0 adds the tag words,
+ * tile offsets and the per-lane escape bytes.  Its duration is the floor the load pattern itself sets under the attention kernel on
+ * the same page.  sink: one uint32 (practically never written). */
+int gaac_read_probe(
+    const uint8_t* smk, const uint8_t* ck, const int* fk, const int* tok, const uint8_t* ovk, const int* ohsk,
+    const uint8_t* smv, const uint8_t* cv, const int* fv, const int* tov, const uint8_t* ovv, const int* ohsv,
+    int H, int S, int S_pad, int nsplit, int with_meta, unsigned int* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
