@@ -77,6 +77,12 @@ __device__ __forceinline__ void store_tile(const PagedStoreArgs& A, EncodeLds& L
       }
     }
   }
+  if (!fits && r < 0 && lane < T) {
+    // side pool exhausted: the slot will read as a compressed tile with stale content (the error counter says so).  Its tag words must
+    // not send a reader past the slot: the size pass above, or an earlier tenant of the block, may have left tags whose escape bytes
+    // (up to 1280) exceed the slot's capacity.  All-zero tags mean no escape bytes.
+    reinterpret_cast<int*>(A.pool + p * A.TS + SLOT_FL)[lane] = 0;
+  }
   if (lane == 0) {
     A.mt[p] = fits || r < 0 ? (int)p : ~r;         // pool exhausted: the slot reads as a (stale) compressed tile, the error counter says so
     A.freeq[qi] = fits && have ? r_old : -1;        // a raw tile that is no longer needed goes back after this launch

@@ -13,9 +13,44 @@ GMAX = 16
 MAX_SPLITS = 1024
 
 
+class _Ext:
+    """What the reference's `_ext()` returns (/root/reference/gaac/kernel.py:332-337): an object whose
+    `gaac_attn_launch(<16 store tensors>, q, slot, n_q, n_kv, SL, S_pad, scale, nsplit, kt, vt, TL, TCAP) -> Tensor` has the tensor
+    signature and behaviour of the reference's pybind entry (kernel.py:296-326): it checks the GQA group and the head dim, allocates the
+    output ([B*n_q, 128], dtype of q), takes the raw tail when `kt.numel() > 0`, launches on the current stream without synchronizing
+    and returns the output.  The calls of /root/reference/gaac/kernel.py:355 and kv_cache.py:188 work on it unchanged.
+    `lib` is the loaded C library (ctypes.CDLL) for callers that want the raw entry points."""
+    def __init__(self, lib):
+        self.lib = lib
+
+    def gaac_attn_launch(self, smk, ck, fk, tok, ovk, ohsk, b3k, b4k, smv, cv, fv, tov, ovv, ohsv, b3v, b4v,
+                         q, slot, n_q, n_kv, SL, S_pad, scale, nsplit, kt, vt, TL, TCAP):
+        G = n_q // max(1, n_kv)
+        if not (1 <= G <= GMAX and G * n_kv == n_q):
+            raise RuntimeError(f"GQA group size must be 1..{GMAX}")
+        if q.shape[-1] != D:
+            raise RuntimeError("head_dim must be 128")
+        B = slot.shape[0]
+        has_tail = kt.numel() > 0
+        out = torch.empty(B * n_q, D, dtype=q.dtype, device=q.device)
+        ws = shared_workspace(B * n_q, nsplit, q.dtype, q.device)
+        p = _lib.ptr
+        _lib.call("gaac_attn_fused", p(smk), p(ck), p(fk), p(tok), p(ovk), p(ohsk), p(b3k), p(b4k),
+                  p(smv), p(cv), p(fv), p(tov), p(ovv), p(ohsv), p(b3v), p(b4v),
+                  p(q), p(slot), B, n_q, n_kv, p(SL), int(S_pad), float(scale), int(nsplit), b3k.shape[0],
+                  p(kt) if has_tail else None, p(vt) if has_tail else None, p(TL) if has_tail else None, int(TCAP) if has_tail else 0,
+                  -1, p(ws.pm), p(ws.pl), p(ws.pa), p(ws.epoch), p(out), _lib.stream())
+        return out
+
+
+_ext_obj = None
+
+
 def _ext():
-    """The loaded native library (raises if it is not built)."""
-    return _lib.load()
+    """The native extension in the shape of the reference's (raises if the library is not built)."""
+    global _ext_obj
+    if _ext_obj is None: _ext_obj = _Ext(_lib.load())
+    return _ext_obj
 
 
 def choose_nsplit(B: int, n_kv: int, S: int, target_ctas: int = 256, min_tok: int = 256, cap: int = 256) -> int:

@@ -110,6 +110,48 @@ def test_launch_shapes_that_share_a_workspace_do_not_mix_their_records():
             assert np.abs(out - ref).max() <= 2e-2 * np.abs(ref).max() + 1e-3
 
 
+def test_native_entry_called_the_way_the_reference_calls_it():
+    """`_ext().gaac_attn_launch(...)` with the reference's tensor arguments, once as /root/reference/gaac/kernel.py:345-358 calls it (two
+    Pages, a slot map 0..B-1, empty tail tensors) and once as /root/reference/gaac/kv_cache.py:183-192 does (cache stores, slot map with a
+    padded row, the raw tails): the output is allocated inside and returned, and matches the oracle."""
+    dev = require_gpu()
+    from gaac_amd.kernel import _ext, choose_nsplit
+    from gaac_amd import CompressedKVCache
+    B, n_kv, G, S = 2, 2, 4, 333
+    n_q = n_kv * G
+    k16, v16, kp, vp = _pages(B, n_kv, S, dev, seed=41)
+    q16 = randn_bf16((B, n_q, 128), seed=42, scale=0.1)
+    q = to_bf16(q16, dev)
+    slots = torch.arange(B, dtype=torch.int32, device=dev)
+    SL = torch.full((kp.H,), kp.S, dtype=torch.int32, device=dev)
+    e = torch.empty(0, dtype=torch.int32, device=dev); eq = torch.empty(0, dtype=q.dtype, device=dev)
+    out = _ext().gaac_attn_launch(kp.sm, kp.codes, kp.flags, kp.tile_off, kp.ovf, kp.ovf_head_start, kp.base3, kp.base4,
+                                  vp.sm, vp.codes, vp.flags, vp.tile_off, vp.ovf, vp.ovf_head_start, vp.base3, vp.base4,
+                                  q.reshape(B * n_q, 128).contiguous(), slots, n_q, n_kv, SL, kp.sm.shape[1] // 128,
+                                  SCALE, choose_nsplit(B, n_kv, kp.S), eq, eq, e, 0)
+    assert out.shape == (B * n_q, 128) and out.dtype == torch.bfloat16
+    got = O.bf16_to_f32(to_u16(out)).reshape(B, n_q, 128); ref = _ref(q16, k16, v16, B, n_kv)
+    assert np.abs(got - ref).max() <= 2e-2 * np.abs(ref).max() + 1e-3
+    # the cache's call: stores with strides of the capacity, lengths and tails on the device, one padded row
+    cache = CompressedKVCache(n_slots=3, n_kv=n_kv, capacity=512)
+    L = 40
+    kt_, vt_ = np.ascontiguousarray(k16[:n_kv, :L].transpose(1, 0, 2)), np.ascontiguousarray(v16[:n_kv, :L].transpose(1, 0, 2))
+    cache.prefill(2, to_bf16(kt_, dev), to_bf16(vt_, dev))
+    sl = torch.tensor([2, -1], dtype=torch.int32, device=dev)
+    K, V = cache.k, cache.v
+    out = _ext().gaac_attn_launch(K.sm, K.codes, K.flags, K.tile_off, K.ovf, K.head_start, K.base3, K.base4,
+                                  V.sm, V.codes, V.flags, V.tile_off, V.ovf, V.head_start, V.base3, V.base4,
+                                  q.reshape(B * n_q, 128).contiguous(), sl, n_q, n_kv, cache.S, cache.cap, SCALE, 3,
+                                  K.tail, V.tail, cache.tail_len, 16)
+    got = O.bf16_to_f32(to_u16(out)).reshape(B, n_q, 128)
+    ref = O.ref_attention(q16[0], kt_, vt_, SCALE)
+    assert np.abs(got[0] - ref).max() <= 2e-2 * np.abs(ref).max() + 1e-3 and np.abs(got[1]).max() == 0
+    with pytest.raises(RuntimeError, match="GQA"):
+        _ext().gaac_attn_launch(K.sm, K.codes, K.flags, K.tile_off, K.ovf, K.head_start, K.base3, K.base4,
+                                V.sm, V.codes, V.flags, V.tile_off, V.ovf, V.head_start, V.base3, V.base4,
+                                q.reshape(B * n_q, 128).contiguous(), sl, n_q, 3, cache.S, cache.cap, SCALE, 3, K.tail, V.tail, cache.tail_len, 16)
+
+
 @pytest.mark.parametrize("B,n_kv,G,S", [(1, 8, 4, 4096), (2, 2, 16, 1000), (3, 2, 1, 16), (1, 4, 6, 333)])
 def test_uncompressed_baseline_kernel(B, n_kv, G, S):
     """The BF16 baseline kernel (same structure, no decoder) against the same oracle and tolerance."""

@@ -125,3 +125,95 @@ def test_byte_offsets_beyond_4_gib():
         ref = torch.einsum("hgs,hsd->hgd", torch.softmax(s, -1), vb).reshape(n_kv * g_, D)
         assert float((out[b] - ref).abs().max()) <= 2e-2 * float(ref.abs().max()) + 1e-3, b
         del kb, vb, s
+
+
+def test_config_2_at_full_size():
+    """24 query heads over 4 kv heads (group 6), 65536 compressed tokens + 7 tail tokens, V's channel scales over 4 octaves, at the
+    launcher's own split count (64 splits of eight-wave blocks) and at others, against fp32 attention on the device over the same rows."""
+    dev = require_gpu()
+    from gaac_amd import Codec, TileEncoder
+    from gaac_amd.kernel import attn_launch, choose_nsplit
+    n_kv, g_ = 4, 6
+    gen = torch.Generator(device=dev).manual_seed(41)
+    def make(spread):
+        sig = torch.exp2(torch.rand(n_kv, 1, D, generator=gen, device=dev) * spread - spread / 2)
+        x = torch.randn(n_kv, S + TAIL, D, generator=gen, device=dev) * sig
+        hit = torch.rand(n_kv, S + TAIL, D, generator=gen, device=dev) < 0.0003
+        return torch.where(hit, x * 4096.0, x).to(torch.bfloat16)
+    k, v = make(2.0), make(4.0)
+    kp = TileEncoder("k").encode(Codec(n_kv).calibrate(k[:, :1024]), k[:, :S].contiguous())
+    vp = TileEncoder("v").encode(Codec(n_kv).calibrate(v[:, :1024]), v[:, :S].contiguous())
+    assert torch.equal(Codec.decode(vp).view(torch.int16), v[:, :S].contiguous().view(torch.int16))
+    q = (torch.randn(n_kv * g_, D, generator=gen, device=dev) * 0.3).to(torch.bfloat16)
+    kt = torch.zeros(n_kv, 16, D, dtype=torch.bfloat16, device=dev); vt = torch.zeros_like(kt)
+    kt[:, :TAIL] = k[:, S:]; vt[:, :TAIL] = v[:, S:]
+    TL = torch.full((n_kv,), TAIL, dtype=torch.int32, device=dev); SL = torch.full((n_kv,), S, dtype=torch.int32, device=dev)
+    s = torch.einsum("hgd,hsd->hgs", q.float().view(n_kv, g_, D), k.float()) * SCALE
+    ref = torch.einsum("hgs,hsd->hgd", torch.softmax(s, -1), v.float()).reshape(n_kv * g_, D)
+    mag = float(ref.abs().max())
+    assert choose_nsplit(1, n_kv, S) == 64
+    for ns, s_all in ((64, S), (64, -1), (32, S), (200, -1)):
+        o = attn_launch(kp, vp, q, None, n_kv * g_, n_kv, SL, S, SCALE, ns, kt, vt, TL, 16, S_all=s_all).float()
+        assert float((o - ref).abs().max()) <= 2e-2 * mag + 1e-3, (ns, s_all)
+        assert float((o - ref).abs().mean()) <= 1e-3 * max(mag, 1.0), (ns, s_all)
+
+
+def test_config_3_paged_pool_at_full_size():
+    """16 sequences of U[4096, 65536] tokens (seed 4) in a pool addressed through a permuted block table (seed 5), 32 query / 8 kv heads:
+    prompts stored, a few decode steps appended (blocks fill up and are compressed), then decode attention at the launcher's split count
+    and at one small enough that the longest sequence puts 1024 tiles into a split (the most a block keeps in its table), against fp32
+    attention on the device over the rows that went in; decode_blocks returns those rows bit for bit."""
+    dev = require_gpu()
+    from gaac_amd.codec import exponent_hist, bases_from_hist
+    from gaac_amd.paged import LayerState, build_store_entries, choose_nsplit, BLOCK
+    n_seq, n_kv, g_, steps = 16, 8, 4, 5
+    n_q = n_kv * g_
+    lens = np.random.default_rng(4).integers(4096, 65537, n_seq).tolist()
+    lens[3] = 65536 - steps                       # one sequence ends exactly on the 1024-tiles-per-split edge at 4 splits
+    nblk = [-(-(L + steps) // BLOCK) for L in lens]
+    perm = np.random.default_rng(5).permutation(sum(nblk))
+    bt_cpu = np.zeros((n_seq, max(nblk)), np.int32); o = 0
+    for i, nb in enumerate(nblk):
+        bt_cpu[i, :nb] = perm[o:o + nb]; o += nb
+    gen = torch.Generator(device=dev).manual_seed(6)
+    sig_k = torch.exp2(torch.rand(1, n_kv, D, generator=gen, device=dev) * 2 - 1); sig_v = torch.exp2(torch.rand(1, n_kv, D, generator=gen, device=dev) * 2 - 1)
+    def rows(n, sig):
+        x = torch.randn(n, n_kv, D, generator=gen, device=dev) * sig
+        hit = torch.rand(n, n_kv, D, generator=gen, device=dev) < 0.0003
+        return torch.where(hit, x * 4096.0, x).to(torch.bfloat16)
+    k3, k4 = bases_from_hist(exponent_hist(rows(1024, sig_k), n_kv), n_kv); v3, v4 = bases_from_hist(exponent_hist(rows(1024, sig_v), n_kv), n_kv)
+    st = LayerState(sum(nblk), n_kv, 2 * n_kv * 4 * n_seq + sum(nblk) * 2 * n_kv // 100 + 64, dict(k3=k3, k4=k4, v3=v3, v4=v4), 128, dev)
+    buf = torch.zeros(LayerState.pool_bytes(sum(nblk), n_kv, 128), dtype=torch.uint8, device=dev)
+    hist_k, hist_v = [], []
+    for i, L in enumerate(lens):
+        kk, vv = rows(L, sig_k), rows(L, sig_v)
+        st.store(kk, vv, buf, torch.from_numpy(build_store_entries([0], [L], [bt_cpu[i]])).to(dev))
+        hist_k.append(kk); hist_v.append(vv)
+    cur = list(lens)
+    for _ in range(steps):
+        kn, vn = rows(n_seq, sig_k), rows(n_seq, sig_v)
+        st.store(kn, vn, buf, torch.from_numpy(build_store_entries(cur, [1] * n_seq, bt_cpu)).to(dev))
+        for i in range(n_seq):
+            hist_k[i] = torch.cat([hist_k[i], kn[i:i + 1]]); hist_v[i] = torch.cat([hist_v[i], vn[i:i + 1]])
+        cur = [c + 1 for c in cur]
+    st.check()
+    bt = torch.from_numpy(bt_cpu).to(dev)
+    seq_lens = torch.tensor(cur, dtype=torch.int32, device=dev)
+    q = (torch.randn(n_seq, n_q, D, generator=gen, device=dev) * 0.3).to(torch.bfloat16)
+    refs = []
+    for i in range(n_seq):
+        s = torch.einsum("hgd,shd->hgs", q[i].float().view(n_kv, g_, D), hist_k[i].float()) * SCALE
+        refs.append(torch.einsum("hgs,shd->hgd", torch.softmax(s, -1), hist_v[i].float()).reshape(n_q, D))
+    assert max(cur) == 65536
+    for ns in (choose_nsplit(n_seq, n_kv, max(cur)), 4, 7):
+        out = st.attention(q, buf, bt, seq_lens, ns, max_seq_len=max(cur)).float().view(n_seq, n_q, D)
+        for i in range(n_seq):
+            assert float((out[i] - refs[i]).abs().max()) <= 2e-2 * float(refs[i].abs().max()) + 1e-3, (ns, i, cur[i])
+    with pytest.raises(RuntimeError, match="max_seq_len"):
+        st.attention(q, buf, bt, seq_lens, 3, max_seq_len=max(cur))      # 4096 tiles in 3 splits: more than a block's table holds
+    for i in (int(np.argmax(cur)), int(np.argmin(cur))):
+        nb_l = -(-cur[i] // BLOCK)
+        pairs = torch.tensor([(int(bt_cpu[i][j]), 16 * j, min(16, cur[i] - 16 * j)) for j in range(nb_l)], dtype=torch.int32, device=dev)
+        sk = torch.empty(cur[i], n_kv, D, dtype=torch.bfloat16, device=dev); sv = torch.empty_like(sk)
+        st.decode_blocks(buf, pairs, sk, sv)
+        assert torch.equal(sk.view(torch.int16), hist_k[i].view(torch.int16)) and torch.equal(sv.view(torch.int16), hist_v[i].view(torch.int16))

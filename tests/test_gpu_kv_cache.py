@@ -211,3 +211,30 @@ def test_many_rows_with_short_and_tail_only_sequences():
         dk, dv = cache.decompress(s)
         assert np.array_equal(to_u16(dk), hist[s][0]) and np.array_equal(to_u16(dv), hist[s][1])
     cache.check_capacity()
+
+
+@pytest.mark.parametrize("per_sequence_bases", [True, False])
+def test_bytes_per_slot_is_what_the_cache_allocates(per_sequence_bases):
+    """bytes_per_slot (/root/reference/gaac/kv_cache.py:142-146) against the tensors a cache really holds: the bytes of every
+    per-head tensor of both stores (tile rows, tag words, tile offsets, escape streams, stream starts, counters, raw tails, and for
+    per-sequence calibration the base rows) plus the two length vectors add up to n_slots * bytes_per_slot, except for the one closing
+    entry of each store's stream-start vector (2 x 4 bytes per cache); per-model base tables (not per slot) are left out, as in the
+    reference's formula.  The oracle's restatement of the formula gives the same number."""
+    dev = require_gpu()
+    from gaac_amd import CompressedKVCache
+    from gaac_amd.codec import exponent_hist, bases_from_hist
+    for (n_slots, n_kv, cap, ovf) in [(1, 1, 16, 128), (3, 2, 1000, 128), (5, 8, 4096, 512), (2, 4, 65536, 64)]:
+        bases = None
+        if not per_sequence_bases:
+            x = to_bf16(np.ascontiguousarray(kv_like16(n_kv, 256, seed=1).transpose(1, 0, 2)), dev)
+            b3, b4 = bases_from_hist(exponent_hist(x, n_kv), n_kv)
+            bases = dict(k3=b3, k4=b4, v3=b3, v4=b4)
+        c = CompressedKVCache(n_slots, n_kv, cap, bases=bases, ovf_bytes_per_tile=ovf)
+        nbytes = lambda t: t.numel() * t.element_size()
+        total = nbytes(c.S) + nbytes(c.tail_len)
+        for st in (c.k, c.v):
+            total += sum(nbytes(t) for t in (st.sm, st.codes, st.flags, st.tile_off, st.ovf, st.head_start, st.ovf_used, st.tail))
+            if per_sequence_bases: total += nbytes(st.base3) + nbytes(st.base4)
+        want = CompressedKVCache.bytes_per_slot(n_kv, cap, ovf, per_sequence_bases)
+        assert total - 2 * 4 == n_slots * want, (n_slots, n_kv, cap, ovf)
+        assert want == O.bytes_per_slot(n_kv, cap, ovf, per_sequence_bases)

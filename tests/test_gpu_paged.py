@@ -162,6 +162,38 @@ def test_raw_pool_exhaustion_is_counted_not_written():
         P.st.check()
 
 
+def test_full_tile_that_fits_nowhere_leaves_a_slot_that_is_safe_to_read():
+    """A finished tile whose escape bytes exceed the slot, stored while the raw side pool is empty: the error counter goes up and the
+    slot is marked compressed with stale content.  Its tag words must be zero (no escape bytes): the sizing pass had written the real
+    ones, whose 1280 escape bytes would send a reader far past the slot, for the pool's last block past the allocation."""
+    dev = require_gpu()
+    from gaac_amd.paged import LayerState, build_store_entries
+    num_blocks = 4
+    st = LayerState(num_blocks, N_KV, 1, _bases(dev), 128, dev)
+    buf = torch.zeros(LayerState.pool_bytes(num_blocks, N_KV, 128), dtype=torch.uint8, device=dev)
+    st.top.zero_()                                          # an empty side pool
+    rng = np.random.default_rng(5)
+    k16 = (rng.integers(0, 1 << 16, (16, N_KV, 128)) & 0xBFFF).astype(np.uint16)      # random exponents: every group is raw
+    v16 = (rng.integers(0, 1 << 16, (16, N_KV, 128)) & 0xBFFF).astype(np.uint16)
+    last = num_blocks - 1
+    ent = build_store_entries([0], [16], [np.array([last], np.int32)])
+    st.store(to_bf16(k16, dev), to_bf16(v16, dev), buf, torch.from_numpy(ent).to(dev))
+    torch.cuda.synchronize()
+    assert int(st.err) == 2 * N_KV
+    nt = 2 * N_KV
+    mt = st.mt.cpu().numpy()
+    assert np.array_equal(mt[last * nt:(last + 1) * nt], np.arange(last * nt, (last + 1) * nt))
+    slots = buf[:num_blocks * nt * st.TS].view(num_blocks * nt, st.TS)[last * nt:(last + 1) * nt]
+    assert int(slots[:, 2816:2880].max()) == 0              # tag words
+    q = to_bf16(randn_bf16((1, N_KV * G, 128), seed=3, scale=0.1), dev)
+    bt = torch.tensor([[last]], dtype=torch.int32, device=dev); sl = torch.tensor([16], dtype=torch.int32, device=dev)
+    out = st.attention(q, buf, bt, sl, nsplit=1, max_seq_len=16)
+    torch.cuda.synchronize()
+    assert out.shape == (1, N_KV * G * 128)
+    with pytest.raises(RuntimeError, match="raw side pool exhausted"):
+        st.check()
+
+
 def test_bad_arguments_raise():
     dev = require_gpu()
     from gaac_amd.paged import LayerState

@@ -259,3 +259,20 @@ def test_byte_accounting_closed_forms():
     st = O.cache_stats(S_sum=64, tail_sum=8, esc=10, n_kv=4)
     assert st["bytes_used"] == 2 * (64 * 180 + 16 + 8 * 256) + 10 and st["bf16_bytes"] == 72 * 512 and st["tokens"] == 18
     assert O.slot_fits(128) and not O.slot_fits(129) and O.OVF_OFF + 128 == 3008
+
+
+def test_attention_error_bound_covers_the_saved_cancellation_case():
+    """tests/golden/attention_cancellation_case.npz: a kernel output (rounded softmax weights) that the reference's tolerance alone
+    rejects (error 1.46 at |ref| <= 67) and that the elementwise bound of common.attention_error_bound accepts, while a result that is
+    off by a few percent of the attended values is still rejected."""
+    import os
+    from common import attention_error_bound
+    d = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "attention_cancellation_case.npz"))
+    q16, k16, v16, out = d["q16"][0], d["k16"], d["v16"], d["out"][0]
+    ref, tol = attention_error_bound(q16, k16, v16, 128 ** -0.5)
+    err = np.abs(out - ref)
+    assert err.max() > 2e-2 * np.abs(ref).max() + 1e-3          # the reference's tolerance alone does not cover it
+    assert (err <= tol).all()
+    assert tol.max() < 2.0 ** -7 * np.abs(O.bf16_to_f32(v16)).max() / 4      # far tighter than a bound by the largest value
+    rnd = tol - (2e-2 * np.abs(ref).max() + 1e-3)
+    assert not (np.abs((ref + 8 * rnd + 0.1 * np.abs(ref).max()) - ref) <= tol).all()
