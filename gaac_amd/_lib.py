@@ -29,6 +29,7 @@ _SIGNATURES = {
     "gaac_stream_copy": [P, P, c_long, P],
     "gaac_read_probe": [P] * 12 + [c_int, c_int, c_int, c_int, c_int, P, P],
     "gaac_attn_fused": [P] * 16 + [P, P, c_int, c_int, c_int, P, c_int, c_float, c_int, c_int, P, P, P, c_int, c_int, P, P, P, P, P, P],
+    "gaac_attn_fused_static": [P] * 16 + [P, P, c_int, c_int, c_int, P, c_int, c_float, c_int, c_int, P, P, P, c_int, c_int, P, P],
     "gaac_attn_launch": [P] * 16 + [P, P, c_int, c_int, c_int, P, c_int, c_float, c_int, c_int, P, P, P, c_int, P, P, P, P, P],
 }
 

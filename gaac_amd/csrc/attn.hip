@@ -1177,6 +1177,46 @@ extern "C" int gaac_attn_fused(
                          scale, nsplit, NB, kt, vt, TL, TCAP, pm, pl, pa, epoch, out, S_all, stream);
 }
 
+// ---- the one entry point that allocates nothing ------------------------------------------------------------------------------------
+// gaac_attn_fused with its workspace (partial records + epoch word) in a file-scope device array instead of caller memory, for callers
+// that cannot allocate: code under HIP graph capture, tight serving loops.  Every GPU the library runs on holds its own copy of the
+// array (4 MiB) from module load to process end; its address on a device comes from hipGetSymbolAddress, once per device.
+constexpr size_t STATIC_SCRATCH_BYTES = 4u << 20;
+constexpr size_t STATIC_EPOCH_BYTES = 256;                                                  // the epoch word, on a line of its own
+constexpr long STATIC_MAX_RECORD_ROWS = (long)((STATIC_SCRATCH_BYTES - STATIC_EPOCH_BYTES) / ((D + 2) * sizeof(u64)));      // B*n_q*nsplit <= 4032
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];              // zero at module load: epoch 0, no records
+constexpr int STATIC_MAX_DEVICES = 64;
+static void* g_scratch_ptr[STATIC_MAX_DEVICES];      // the array's address on each device (the name `scratch` is not one in host code)
+
+extern "C" int gaac_attn_fused_static(
+    const uint8_t* smk, const uint8_t* ck, const int* fk, const int* tok, const uint8_t* ovk, const int* ohsk, const uint8_t* b3k, const uint8_t* b4k,
+    const uint8_t* smv, const uint8_t* cv, const int* fv, const int* tov, const uint8_t* ovv, const int* ohsv, const uint8_t* b3v, const uint8_t* b4v,
+    const void* q, const int* slot, int B, int n_q, int n_kv, const int* SL, int S_pad, float scale, int nsplit, int NB,
+    const void* kt, const void* vt, const int* TL, int TCAP, int S_all, void* out, void* stream) {
+  GAAC_REQUIRE(out, "gaac_attn_fused_static: null output");
+  GAAC_REQUIRE(B > 0 && n_q > 0 && nsplit >= 1, "gaac_attn_fused_static: bad sizes B=%d n_q=%d nsplit=%d", B, n_q, nsplit);
+  const long rec_rows = (long)B * n_q * nsplit;
+  GAAC_REQUIRE(rec_rows <= STATIC_MAX_RECORD_ROWS,
+               "gaac_attn_fused_static: B*n_q*nsplit = %ld exceeds the %ld partial rows the built-in workspace (%zu bytes) holds; use gaac_attn_fused with caller memory",
+               rec_rows, STATIC_MAX_RECORD_ROWS, STATIC_SCRATCH_BYTES);
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= STATIC_MAX_DEVICES) return gaac::fail("gaac_attn_fused_static: no current device (%s)", hipGetErrorString(e));
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) return gaac::fail("gaac_attn_fused_static: hipGetSymbolAddress failed (%s)", hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  unsigned char* base = static_cast<unsigned char*>(g_scratch_ptr[dev]);
+  unsigned int* epoch = reinterpret_cast<unsigned int*>(base);
+  unsigned long long* pm = reinterpret_cast<unsigned long long*>(base + STATIC_EPOCH_BYTES);
+  unsigned long long* pl = pm + rec_rows;
+  unsigned long long* pa = pl + rec_rows;
+  return attn_split_impl(smk, ck, fk, tok, ovk, ohsk, b3k, b4k, smv, cv, fv, tov, ovv, ohsv, b3v, b4v, q, slot, B, n_q, n_kv, SL, S_pad,
+                         scale, nsplit, NB, kt, vt, TL, TCAP, pm, pl, pa, epoch, out, S_all, stream);
+}
+
 extern "C" int gaac_paged_attn(
     const uint8_t* pool, int TS, const void* raw, const int* mt, const int* bt, int bt_stride, const int* seq_lens, int max_seq_len,
     const void* q, int B, int n_q, int n_kv, float scale, int nsplit,

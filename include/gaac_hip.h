@@ -93,6 +93,18 @@ int gaac_attn_fused(
     const void* kt, const void* vt, const int* TL, int TCAP, int S_all,
     unsigned long long* pm, unsigned long long* pl, unsigned long long* pa, unsigned int* epoch, void* out, void* stream);
 
+/* gaac_attn_fused for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that forbid it): the
+ * same launch, but the partial records and the epoch word live in a 4 MiB array built into the library (one copy per GPU, held from
+ * load to process end) instead of caller memory; the call itself allocates nothing.  It has no counterpart in the reference, whose
+ * entry allocates its partials on every call (kernel.py:306-307).  Limit: B*n_q*nsplit <= 4032 partial rows (the headline launch uses
+ * 1024); larger launches are rejected with -1 and a message.  All calls on one GPU share the array: they must be ordered on one
+ * stream (calls that overlap on a GPU race), and nothing needs clearing between them (the epoch tells launches apart). */
+int gaac_attn_fused_static(
+    const uint8_t* smk, const uint8_t* ck, const int* fk, const int* tok, const uint8_t* ovk, const int* ohsk, const uint8_t* b3k, const uint8_t* b4k,
+    const uint8_t* smv, const uint8_t* cv, const int* fv, const int* tov, const uint8_t* ovv, const int* ohsv, const uint8_t* b3v, const uint8_t* b4v,
+    const void* q, const int* slot, int B, int n_q, int n_kv, const int* SL, int S_pad, float scale, int nsplit, int NB,
+    const void* kt, const void* vt, const int* TL, int TCAP, int S_all, void* out, void* stream);
+
 /* CompressedKVCache.append, /root/reference/gaac/kv_cache.py:172-181 (kernels _append_one/_append_kv/_advance, :22-96), as one
  * launch: row i = b*n_kv + kvh of k_new/v_new [B, n_kv, 128] bf16 goes to tail row tail_len[h] of cache head
  * h = slots[b]*n_kv + kvh (slots[b] < 0: skipped); when that fills the 16-row tail the tile is compressed in place as tile S[h]/16
