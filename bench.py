@@ -484,38 +484,76 @@ def bench_serve(a):
     prompts = [torch.randint(0, cfg.vocab, (ctx,), generator=g, device=dev) for _ in range(B)]
     res = {"workload": f"config 4: Llama-3-8B architecture (random init, bf16), batch {B}, {ctx}-token random contexts, greedy decode, one HIP graph per step",
            "weights_bytes": w.nbytes(), "steps": steps}
-    toks, logits1 = {}, {}
-    for kv in ("gaac", "bf16"):
+    # Teacher forcing first: both runs consume the same FORCED tokens, eagerly, so their per-step logits and cache contents compare
+    # one to one (free-running greedy runs on random weights, whose logits are nearly flat, flip a token on attention rounding and
+    # then drift apart).  The timed region is the free-running decode after it, the whole step replayed as one graph.
+    FORCED = 8
+    forced = torch.randint(0, cfg.vocab, (FORCED, B), generator=g, device=dev)
+
+    def checksum(x, L):      # position-weighted sum of the BF16 bit patterns of rows [0, L) of a [rows, n_kv, D] tensor
+        bits = x[:L].contiguous().view(torch.int16).to(torch.int64).flatten()
+        return int((bits * (torch.arange(bits.numel(), device=dev) % 65521 + 1)).sum().item())
+
+    def forced_run(kv, nsplit=None):
         run = DecodeRunner(w, n_slots=B, kv=kv)
         t0 = time.perf_counter()
         first = torch.stack([run.prefill(i, p).argmax() for i, p in enumerate(prompts)])
         torch.cuda.synchronize(); t_prefill = time.perf_counter() - t0
-        run.start_decode(first, use_graph=True)
-        run.decode(1); logits1[kv] = run.logits.float().clone()
-        run.decode(7); torch.cuda.synchronize()
+        fed = [[] for _ in range(cfg.n_layers)]
+        hooks = [at.register_forward_hook(lambda m, args, out, l=l: fed[l].append((args[1].clone(), args[2].clone()))) for l, at in enumerate(run.attn)]
+        run.start_decode(first, use_graph=False, nsplit=nsplit)
+        _, lg = run.decode(FORCED, forced=forced, keep_logits=True)
+        for h in hooks: h.remove()
+        return run, first, lg, fed, t_prefill
+
+    toks, flogits, sums = {}, {}, {}
+    for kv in ("gaac", "bf16"):
+        run, first, flogits[kv], fed, t_prefill = forced_run(kv)
+        cs = []
+        for l in range(cfg.n_layers):
+            for slot in range(B):
+                L = ctx + FORCED if l == 0 else ctx      # layer 0 sees the same inputs in both runs; deeper layers only during prefill
+                if kv == "gaac":
+                    dk, dv = run.caches[l].decompress(slot)
+                    assert dk.shape[0] == ctx + FORCED
+                    # lossless: the rows appended during the forced steps are bit for bit what the layer was handed
+                    nk = torch.stack([f[0][slot] for f in fed[l]]); nv = torch.stack([f[1][slot] for f in fed[l]])
+                    assert torch.equal(dk[ctx:].view(torch.int16), nk.view(torch.int16)) and torch.equal(dv[ctx:].view(torch.int16), nv.view(torch.int16)), \
+                        f"layer {l} slot {slot}: the compressed cache does not hold the rows it was given"
+                else:
+                    c, h0 = run.caches[l], slot * cfg.n_kv_heads
+                    dk, dv = c.k[h0:h0 + cfg.n_kv_heads, :L].transpose(0, 1), c.v[h0:h0 + cfg.n_kv_heads, :L].transpose(0, 1)
+                cs.append((checksum(dk, L), checksum(dv, L)))
+                del dk, dv
+        sums[kv] = cs
+        run.start_decode(forced[-1], use_graph=True)
+        run.decode(8); torch.cuda.synchronize()
         t0 = time.perf_counter()
         toks[kv] = run.decode(steps)
         torch.cuda.synchronize(); dt = time.perf_counter() - t0
         st = run.kv_stats()
         res[kv] = {"tokens_per_s": round(B * steps / dt, 1), "ms_per_step": round(dt / steps * 1e3, 3), "prefill_s": round(t_prefill, 2),
                    "kv_bytes_used": st["bytes_used"], "kv_bytes_reserved": st["bytes_reserved"], "kv_ratio_vs_bf16": round(st["ratio"], 4)}
-        del run
+        del run, fed
         torch.cuda.empty_cache()
-    # noise floor: the uncompressed run again with another split count (same kernel, another summation order)
-    run = DecodeRunner(w, n_slots=B, kv="bf16")
-    first = torch.stack([run.prefill(i, p).argmax() for i, p in enumerate(prompts)])
-    run.start_decode(first, use_graph=False, nsplit=5)
-    run.decode(1)
-    dn = (run.logits.float() - logits1["bf16"]).abs()
+    assert sums["gaac"] == sums["bf16"], "cache contents differ between the compressed and the uncompressed run"
+    # noise floor: the uncompressed run again with another split count (same kernel, same forced tokens, another summation order)
+    run, _, ln, _, _ = forced_run("bf16", nsplit=5)
     del run
-    # the cache is lossless, so both runs see the same K/V; they differ by the rounding of two different attention kernels.  With random
-    # weights the logits are nearly flat, so greedy tokens flip on that rounding and the runs then drift apart: the first step's logits
-    # are the meaningful comparison
-    d = (logits1["gaac"] - logits1["bf16"]).abs()
-    res["first_step_logits"] = {"max_abs_diff": round(d.max().item(), 5), "mean_abs_diff": round(d.mean().item(), 6),
-                                "logit_std": round(logits1["bf16"].std().item(), 4),
-                                "noise_floor_max_abs_diff": round(dn.max().item(), 5), "noise_floor_mean_abs_diff": round(dn.mean().item(), 6),
-                                "same_argmax_rows": int((logits1["gaac"].argmax(-1) == logits1["bf16"].argmax(-1)).sum().item())}
+    torch.cuda.empty_cache()
+    d = (flogits["gaac"] - flogits["bf16"]).abs().flatten(1)      # [FORCED, B * vocab]
+    dn = (ln - flogits["bf16"]).abs().flatten(1)
+    # the cache is lossless, so both runs see the same K/V; they differ by the rounding of two different attention kernels, which 32
+    # layers of random weights amplify: the bar is a small multiple of what a mere change of summation order does to the same model
+    for i in range(FORCED):
+        assert d[i].max().item() <= 4 * dn.max().item() and d[i].mean().item() <= 2 * dn.mean().item(), \
+            f"forced step {i}: logits differ by max {d[i].max().item():.4g} / mean {d[i].mean().item():.4g}; noise floor max {dn.max().item():.4g} / mean {dn.mean().item():.4g}"
+    res["teacher_forced"] = {"steps": FORCED, "cache_contents": "bit-identical (position-weighted checksums of K and V, every layer and sequence; appended rows compared bit for bit)",
+                             "logits_max_abs_diff_per_step": [round(x, 5) for x in d.max(1).values.tolist()],
+                             "logits_mean_abs_diff_per_step": [round(x, 6) for x in d.mean(1).tolist()],
+                             "logit_std": round(flogits["bf16"].std().item(), 4),
+                             "noise_floor_max_abs_diff": round(dn.max().item(), 5), "noise_floor_mean_abs_diff": round(dn.mean().item(), 6),
+                             "same_argmax_fraction": round((flogits["gaac"].argmax(-1) == flogits["bf16"].argmax(-1)).float().mean().item(), 4)}
     res["same_tokens_fraction"] = round((toks["gaac"] == toks["bf16"]).float().mean().item(), 4)
     res["speedup"] = round(res["gaac"]["tokens_per_s"] / res["bf16"]["tokens_per_s"], 4)
     print(json.dumps(res))
