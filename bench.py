@@ -578,16 +578,16 @@ def bench_phases(a):
     kt = torch.zeros(H, 16, D, dtype=torch.bfloat16, device=dev); vt = torch.zeros_like(kt)
     kt[:, :TAIL_TOK] = kd[:, S_CTX:]; vt[:, :TAIL_TOK] = vd[:, S_CTX:]
     TL = torch.full((H,), TAIL_TOK, dtype=torch.int32, device=dev); SL = torch.full((H,), S_CTX, dtype=torch.int32, device=dev)
-    slots = torch.zeros(1, dtype=torch.int32, device=dev)
     q2d = torch.randn(n_q, D, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16).to(dev)
     nsplit = a.nsplit or choose_nsplit(1, N_KV, S_CTX)
     nblk = H * nsplit
     NW = 8 if nblk <= 256 else 4
     ws = AttnWorkspace(n_q, nsplit, torch.bfloat16, dev)
-    dbg = torch.zeros(nblk * 16, dtype=torch.int64, device=dev)
+    STAMPS = 32      # int64 per block: 8 block stamps | 8 per-wave loop ends | 8 merge stamps (three planes of nblk * 8), rounded up
+    dbg = torch.zeros(nblk * STAMPS, dtype=torch.int64, device=dev)
     lib = _lib.load(); lib.gaac_set_phase_buffer.argtypes = [ctypes.c_void_p]; lib.gaac_set_phase_buffer.restype = None
     lib.gaac_set_phase_buffer(dbg.data_ptr())
-    f = lambda i: attn_launch(pages[i % len(pages)][0], pages[i % len(pages)][1], q2d, None if os.environ.get("PH_SALL") else slots, n_q, N_KV, SL, S_CTX, D ** -0.5, nsplit, kt, vt, TL, 16, ws=ws, S_all=S_CTX if os.environ.get("PH_SALL") else -1)
+    f = lambda i: attn_launch(pages[i % len(pages)][0], pages[i % len(pages)][1], q2d, None, n_q, N_KV, SL, S_CTX, D ** -0.5, nsplit, kt, vt, TL, 16, ws=ws, S_all=S_CTX)      # the launch the attn workload times
     for i in range(10): f(i)
     rows = []
     for i in range(20):
@@ -595,18 +595,21 @@ def bench_phases(a):
         raw = dbg.cpu().numpy().astype(np.float64) * 0.01          # us
         t = raw[:nblk * 8].reshape(nblk, 8); t0 = t[:, 0].min()
         main = t - t0
-        wv = raw[nblk * 8:].reshape(nblk, 8)[:, :NW] - t0
+        wv = raw[nblk * 8:nblk * 16].reshape(nblk, 8)[:, :NW] - t0
+        mg = raw[nblk * 16:nblk * 24].reshape(nblk, 8); mg = mg[mg[:, 0] > 0] - t0      # blocks that merged (their last half head)
         xcd = np.arange(nblk) % 8
         ends = wv.max(1)
         rows.append([main[:, 0].max(), main[:, 6].mean(), main[:, 1].mean(), wv[:, :4].mean(), wv[:, NW - 4:].mean(), ends.mean(), ends.max(),
-                     main[:, 4].mean(), main[:, 4].max(), (t[:, 5] - t0).max(), min(ends[xcd == x].mean() for x in range(8)), max(ends[xcd == x].mean() for x in range(8))])
+                     main[:, 4].mean(), main[:, 4].max(), (t[:, 5] - t0).max(), min(ends[xcd == x].mean() for x in range(8)), max(ends[xcd == x].mean() for x in range(8)),
+                     mg[:, 0].max(), mg[:, 1].max(), mg[:, 2].max(), mg[:, 4].max()])
     m = np.median(np.array(rows), 0)
     names = ["last_block_start", "first_tile_loads_issued_mean", "tables_ready_mean", "loop_end_waves_0_3_mean", f"loop_end_waves_{NW - 4}_{NW - 1}_mean",
-             "block_loop_end_mean", "block_loop_end_max", "partial_stored_mean", "partial_stored_max", "last_stamp", "loop_end_fastest_xcd_mean", "loop_end_slowest_xcd_mean"]
+             "block_loop_end_mean", "block_loop_end_max", "partial_stored_mean", "partial_stored_max", "last_stamp", "loop_end_fastest_xcd_mean", "loop_end_slowest_xcd_mean",
+             "merge_first_reads_issued_max", "merge_records_all_arrived_max", "merge_weighted_sum_done_max", "merge_output_stored_max"]
     # the same launches back to back (one HIP graph, a stamp buffer per launch): what the idle gap between dependent launches is and
     # how the phases move when arguments and metadata are still cached from the launch before
     nb2b = 24
-    dbgs = torch.zeros(nb2b, nblk * 16, dtype=torch.int64, device=dev)
+    dbgs = torch.zeros(nb2b, nblk * STAMPS, dtype=torch.int64, device=dev)
     def chain():
         for i in range(nb2b):
             lib.gaac_set_phase_buffer(dbgs[i].data_ptr()); f(i)
@@ -619,7 +622,7 @@ def bench_phases(a):
     for _ in range(5):
         dbgs.zero_(); torch.cuda.synchronize(); g.replay(); torch.cuda.synchronize()
         raw = dbgs.cpu().numpy().astype(np.float64) * 0.01
-        t = raw[:, :nblk * 8].reshape(nb2b, nblk, 8); wv = raw[:, nblk * 8:].reshape(nb2b, nblk, 8)[:, :, :NW]
+        t = raw[:, :nblk * 8].reshape(nb2b, nblk, 8); wv = raw[:, nblk * 8:nblk * 16].reshape(nb2b, nblk, 8)[:, :, :NW]
         first, last = t[:, :, 0].min(1), t[:, :, 5].max(1)
         for i in range(4, nb2b - 1):
             b2b.append([first[i + 1] - first[i], first[i + 1] - last[i], last[i] - first[i], (t[i, :, 1] - first[i]).mean(),

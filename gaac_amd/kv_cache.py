@@ -1,12 +1,17 @@
-"""Compressed KV cache of one attention layer for serving on MI355X.
+"""Slot-based compressed KV cache of one attention layer, resident in HBM, behind the interface of
+/root/reference/gaac/kv_cache.py:122-234 (constructor arguments, method names, attribute names and tensor shapes are that
+class's, so an engine written against it runs unchanged).
 
-Drop-in for the cache of /root/reference/gaac/kv_cache.py:122-234 (same constructor, methods, attributes and tensor
-shapes).  A sequence owns a slot of n_kv cache heads; a head stores compressed 16-token tiles (token stride `cap`), one
-escape stream of `ovf_cap` bytes and a raw BF16 tail of 0..15 tokens.  A decode step is two launches on the current
-stream, append (the step that fills a tail compresses the tile in place) and attention, without host synchronization,
-so it can be captured in a HIP graph; batch rows find their slot through a device slot map and rows with slot -1 are
-skipped (attention output exactly 0).  Bases are per model ([n_kv, D] tables) or per sequence, calibrated on the
-prompt at prefill ([n_slots*n_kv, D] tables)."""
+Layout: slot s owns cache heads [s*n_kv, (s+1)*n_kv).  Per head and kind there are `cap` token rows of compressed tiles
+(16 tokens each), a fixed window of `ovf_cap` bytes in the escape buffer, and a 16-row BF16 staging tail that collects
+tokens until a tile is complete.  A decode step costs two launches on the current stream and never returns to the host:
+`append` writes one token per batch row (and encodes the tile in place on the step that completes it), `attention` reads
+tiles + tail.  Both take the batch's slot map from device memory, so the step can be captured in a HIP graph; a row whose
+slot is -1 is left alone (its attention output is exactly 0).  Exponent bases come either from the caller ([n_kv, D],
+shared by all sequences) or from each prompt at prefill ([n_slots*n_kv, D]).
+
+The escape buffers carry 8 bytes of padding behind the last head's window, because the kernels fetch escape bytes with
+unaligned 8-byte loads that may reach past a head's last escape byte; bytes_per_slot counts that padding per head."""
 from __future__ import annotations
 import torch
 from . import _lib
@@ -24,7 +29,7 @@ def _round_up_tokens(n: int) -> int:
 
 
 class _Store:
-    """One kind ('k' | 'v') of the cache: the tensors the kernels read, named as in kv_cache.py:99-111."""
+    """The K half or the V half of the cache.  Attribute names are those of kv_cache.py:99-111, which the attention launch reads by name."""
     def __init__(self, kind: str, H: int, cap: int, ovf_cap: int, base3: torch.Tensor, base4: torch.Tensor, dev):
         z = lambda *shape, dtype=torch.uint8: torch.zeros(*shape, dtype=dtype, device=dev)
         self.kind, self.H, self.cap = kind, H, cap
@@ -42,20 +47,20 @@ class _Store:
         self.head_start = (torch.arange(self.H + 1, device=buf.device, dtype=torch.int32) * ovf_cap).contiguous()
 
     def grow(self, ovf_cap: int):
-        """Re-home every head's escape bytes in a stream of ovf_cap bytes per head."""
+        """Move to an escape buffer with ovf_cap bytes per head, keeping every head's bytes at the start of its new window."""
         wider = torch.zeros(self.H * ovf_cap, dtype=torch.uint8, device=self.ovf.device)
         wider.view(self.H, ovf_cap)[:, :self.ovf_cap].copy_(self.ovf.view(self.H, self.ovf_cap))
         self._set_stream(wider, ovf_cap)
 
     def heads(self, h0: int, h1: int, S: int, n_kv: int) -> Page:
-        """The compressed part of heads [h0, h1) as a Page view (no copies)."""
+        """Page over the tiles of heads [h0, h1), S tokens each; shares the cache's memory."""
         own_rows = self.base3.shape[0] != n_kv
         b3, b4 = (self.base3[h0:h1], self.base4[h0:h1]) if own_rows else (self.base3, self.base4)
         return Page(self.sm[h0:h1], self.codes[h0:h1], self.flags[h0:h1], row_offsets(self.flags[h0:h1], S), self.ovf,
                     self.head_start[h0:h1 + 1], self.tile_off[h0:h1], b3, b4, h1 - h0, S, n_kv, self.kind)
 
     def load_prompt(self, h0: int, h1: int, xh: torch.Tensor, n_kv: int, calibrate: bool, grow) -> None:
-        """xh: [n_kv, L, D] (any strides).  Full tiles are compressed into rows [0, L//16*16) of the heads, the rest becomes the tail."""
+        """xh: [n_kv, L, D], any strides.  The first L - L % 16 tokens are encoded into the heads' tile rows; the remaining L % 16 go to the tail raw."""
         L = xh.shape[1]; full = L // T * T
         if calibrate:
             c = Codec(n_kv, xh.device).calibrate(xh)
@@ -79,8 +84,9 @@ class _Store:
 class CompressedKVCache:
     def __init__(self, n_slots: int, n_kv: int, capacity: int, bases: dict | None = None,
                  ovf_bytes_per_tile: int = 128, device="cuda"):
-        """capacity: max tokens per sequence; bases: {'k3','k4','v3','v4'} uint8 [n_kv, D] (None = per-sequence calibration);
-        ovf_bytes_per_tile: escape-stream reservation per 16-token tile."""
+        """n_slots sequences of up to `capacity` tokens (rounded up to whole tiles), n_kv cache heads each.  bases: dict with uint8
+        [n_kv, D] tables under 'k3', 'k4', 'v3', 'v4', or None to calibrate on every prompt.  ovf_bytes_per_tile sizes each head's
+        escape window: that many bytes for every tile the head can hold (the window grows on demand until a graph is captured)."""
         _ext()      # fail here, not at the first decode step, if the native library is missing
         self.n_slots, self.n_kv = n_slots, n_kv
         self.cap = _round_up_tokens(capacity)
@@ -101,8 +107,10 @@ class CompressedKVCache:
 
     @staticmethod
     def bytes_per_slot(n_kv: int, capacity: int, ovf_bytes_per_tile: int = 128, per_sequence_bases: bool = True) -> int:
-        """Resident bytes of one slot (kv_cache.py:142-146): per head and kind the tile rows, tile offsets, escape stream
-        (+8 padding), two counters, the raw tail and, for per-sequence bases, two base rows; plus S and tail_len per head."""
+        """Device bytes one slot occupies, the quantity an engine divides its memory budget by (kv_cache.py:142-146).  Per head,
+        for K and for V: token rows (sign/mantissa + codes + tag word), one offset per tile, the escape window and its 8 bytes of
+        read padding, the escape counter (8 bytes with alignment), the staging tail, and with per-sequence bases the two base
+        rows; per head once more: the S and tail_len counters."""
         cap = _round_up_tokens(capacity); tiles = cap // T
         head = cap * ROW_BYTES + tiles * 4 + (tiles * ovf_bytes_per_tile + 8) + 8 + TAIL * D * 2
         if per_sequence_bases: head += 2 * D
@@ -110,9 +118,9 @@ class CompressedKVCache:
 
     # ------------------------------------------------------------------ prefill
     def prefill(self, slot: int, k: torch.Tensor, v: torch.Tensor):
-        """Store a sequence's prompt K/V ([L, n_kv, D] bf16, token-major as produced by the model) in `slot` (a reused slot is reset)."""
+        """Put a whole prompt into `slot`, replacing what the slot held: k, v bf16 [L, n_kv, D] in the model's token-major layout."""
         L = k.shape[0]
-        assert L <= self.cap, f"sequence of {L} tokens exceeds the cache capacity {self.cap}"
+        assert L <= self.cap, f"prompt has {L} tokens, a slot holds {self.cap}"
         h0, h1 = slot * self.n_kv, (slot + 1) * self.n_kv
         for st, x in ((self.k, k), (self.v, v)):
             st.load_prompt(h0, h1, x.contiguous().transpose(0, 1), self.n_kv, self.per_sequence_bases, self._grow)      # a view: no transposing copy
@@ -121,7 +129,8 @@ class CompressedKVCache:
 
     # ------------------------------------------------------------------ decode step
     def append(self, slots: torch.Tensor, k: torch.Tensor, v: torch.Tensor):
-        """One new token per batch row: slots int32 [B] (-1 = skip), k/v [B, n_kv, D] bf16.  One launch, graph-safe."""
+        """Decode-step write: batch row b adds the token k[b], v[b] (bf16 [B, n_kv, D]) to slot slots[b] (int32 [B]; -1 leaves the row out).
+        A single launch with no host synchronization."""
         k, v = k.contiguous(), v.contiguous()
         if k.dtype != torch.bfloat16 or v.dtype != torch.bfloat16 or k.shape != v.shape or tuple(k.shape[1:]) != (self.n_kv, D):
             raise RuntimeError(f"append expects k, v bf16 [B, {self.n_kv}, {D}]")
@@ -132,7 +141,8 @@ class CompressedKVCache:
                   self.k.base3.shape[0], *self.k.kernel_args(), *self.v.kernel_args(), p(self.overflow), _lib.stream())
 
     def attention(self, q: torch.Tensor, slots: torch.Tensor, scale: float, max_len: int | None = None, nsplit: int | None = None):
-        """q: [B, n_q, D] bf16 (row b attends over slot slots[b]) -> [B, n_q, D] bf16."""
+        """Decode-step read: bf16 [B, n_q, D] queries, row b over everything slot slots[b] holds (tiles and tail); returns bf16 [B, n_q, D].
+        max_len only picks the split count when nsplit is not given."""
         B, n_q, _ = q.shape
         if nsplit is None: nsplit = choose_nsplit(B, self.n_kv, max_len or self.cap)
         ws = self._partials.get((B, n_q, nsplit))
@@ -147,24 +157,26 @@ class CompressedKVCache:
         return torch.maximum(self.k.ovf_used.max(), self.v.ovf_used.max())
 
     def check_capacity(self, used: int | None = None):
-        """Call at least once every 16 decode steps: a head finalizes at most one tile in 16 steps, so one worst-case tile of
-        headroom per head keeps the escape streams overflow-proof between checks (kv_cache.py:198-203)."""
+        """Host-side guard of the escape windows (kv_cache.py:198-203); the engine calls it every 16 decode steps at the latest.  In
+        16 steps a head completes one tile at most, and a tile has at most TILE_MAX_ESC escape bytes, so a window that has that
+        much room left after a check cannot fill up before the next one.  Grows the windows when the room is gone; raises if the
+        append kernel already had to drop data.  used: max_escape_bytes() if the caller fetched it already."""
         hit = int(self.overflow)
         if hit:
-            raise RuntimeError("compressed KV cache overflow:" + (" a head exceeded its token capacity;" if hit & 1 else "") +
-                               (" an escape stream was full (check_capacity must run at least every 16 decode steps)" if hit & 2 else ""))
+            raise RuntimeError("compressed KV cache lost data:" + (" a sequence grew past the slot's token capacity;" if hit & 1 else "") +
+                               (" an escape window filled up between two check_capacity calls (call it every 16 decode steps)" if hit & 2 else ""))
         used = int(self.max_escape_bytes()) if used is None else used
         if used + HEADROOM > self.k.ovf_cap: self._grow(used + HEADROOM)
 
     def _grow(self, need: int):
         if not self.growable:
-            raise RuntimeError(f"escape stream needs {need} B per head but holds {self.k.ovf_cap} B and graphs are captured; "
-                               "raise ovf_bytes_per_tile or calibrate the exponent bases on representative prompts")
+            raise RuntimeError(f"every head's escape window must grow from {self.k.ovf_cap} to {need} bytes, but a captured graph holds the "
+                               "buffer's address: construct the cache with a larger ovf_bytes_per_tile, or pass bases calibrated on typical prompts")
         cap = max(2 * self.k.ovf_cap, need + 4096 + 7) // 8 * 8
         self.k.grow(cap); self.v.grow(cap)
 
     def decompress(self, slot: int) -> tuple[torch.Tensor, torch.Tensor]:
-        """Bit-exact BF16 K/V of `slot` ([L, n_kv, D] each): decoded tiles followed by the raw tail."""
+        """The K and V that `slot` holds, bf16 [L, n_kv, D] each, equal bit for bit to what was stored: tiles through the decoder kernel, then the tail rows."""
         h0, h1 = slot * self.n_kv, (slot + 1) * self.n_kv
         S, n_tail = int(self.S[h0]), int(self.tail_len[h0])
         def one(st):
@@ -174,7 +186,8 @@ class CompressedKVCache:
         return one(self.k), one(self.v)
 
     def stats(self) -> dict:
-        """Bytes in use (compressed tiles + escapes + metadata + raw tails) vs the BF16 bytes of the same tokens (kv_cache.py:228-234)."""
+        """Occupancy (same keys as kv_cache.py:228-234): bytes_used counts encoded rows, tile offsets, escape bytes and the BF16 tail rows of
+        all slots; bf16_bytes is what the same tokens take uncompressed."""
         rows, raw_rows = int(self.S.sum()), int(self.tail_len.sum())
         escapes = int(self.k.ovf_used.sum()) + int(self.v.ovf_used.sum())
         used = 2 * (rows * ROW_BYTES + rows // T * 4 + raw_rows * D * 2) + escapes

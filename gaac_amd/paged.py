@@ -43,7 +43,9 @@ def build_store_entries(num_computed, query_len, block_table) -> np.ndarray:
 
 
 class LayerState:
-    """Per-layer device state outside the block pool: raw side pool, mode table, free stack, error counter and bases."""
+    """Per-layer device state outside the block pool: raw side pool, mode table, free stack, error counter and bases.  The block pool
+    itself is the caller's allocation; it must be pool_bytes() long, i.e. reach 16 bytes past its last tile slot (at least 8 are
+    required: the kernels fetch escape bytes with unaligned 8-byte loads that may start at the last byte of a slot)."""
     def __init__(self, num_blocks: int, n_kv: int, raw_tiles: int, bases: dict, ovf_slot: int = 128, device="cuda"):
         _lib.load()
         self.n_kv, self.ovf_slot, self.TS = n_kv, ovf_slot, OVF_OFF + ovf_slot
@@ -120,7 +122,9 @@ class LayerState:
 def paged_attention(q, out, buf, raw, mt, bt, seq_lens, bases, TS, n_q, n_kv, nsplit, max_seq_len=None, ws=None):
     """q: [B, n_q, 128] bf16 contiguous; out: [B, n_q*128] bf16 (written); buf: uint8 flat block pool; raw: [tiles,16,128] bf16;
     mt: int32 [num_blocks*2*n_kv]; bt: int32 [B, max_blocks]; seq_lens: int32 [B]; bases: (b3k,b4k,b3v,b4v) uint8 [n_kv,128].
-    max_seq_len: host-side bound of seq_lens (default: what the block table can address)."""
+    max_seq_len: host-side bound of seq_lens (default: what the block table can address).  buf must extend at least 8 bytes past its
+    last tile slot (LayerState.pool_bytes includes 16): escape bytes are fetched with unaligned 8-byte loads.  ws: the launch's
+    AttnWorkspace (default: one cached per device, stream and launch shape, so repeated calls allocate nothing)."""
     B = q.shape[0]
     if q.shape[-1] != D: raise RuntimeError("head_dim must be 128")
     if max_seq_len is None: max_seq_len = bt.shape[1] * BLOCK

@@ -8,7 +8,10 @@
  *   - BF16 tensors are passed as void* (16-bit patterns); `kind` is 0 for K, 1 for V.
  *
  * Byte order inside a 16-token tile (sign/mantissa and code bytes) is the gfx950 MFMA operand order documented in
- * gaac_amd/csrc/gaac_core.h; tag words, tile offsets and the escape stream have the reference's order.
+ * gaac_amd/csrc/gaac_core.h.  K tag words and K escape bytes have the reference's order (one tag word per token; escapes by
+ * token, then group).  V tag words and V escape bytes are transposed within the tile: tag word a of a tile belongs to GROUP a
+ * and holds the tags of its 16 tokens (token j at bits 2j), and the tile's escape bytes run by group, then token.  Per-tile
+ * escape byte counts, tile offsets and head starts are the reference's numbers.
  * Citations are to the reference interface each entry point replaces.
  */
 #ifndef GAAC_HIP_H

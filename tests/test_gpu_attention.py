@@ -166,6 +166,46 @@ def test_uncompressed_baseline_kernel(B, n_kv, G, S):
             assert np.abs(got[b] - ref[b]).max() <= 2e-2 * np.abs(ref[b]).max() + 1e-3, (b, ns)
 
 
+@pytest.mark.parametrize("kernel", ["compressed", "uncompressed"])
+@pytest.mark.parametrize("B,nsplit", [(1, 6), (3, 11)], ids=["eight_wave_blocks", "four_wave_blocks"])
+@pytest.mark.parametrize("rest", [1, 5, 9, 15])
+def test_scores_of_a_partly_filled_last_tile_are_read_only_after_the_matrix_unit_delivered_them(kernel, B, nsplit, rest):
+    """Regression guard for a hazard between the matrix unit and the vector ALU: the scores of a tile come out of an MFMA, and their
+    first VALU read (masking the tokens past the end, the running maximum) must not start before the MFMA has delivered them.  The
+    hardware does not interlock that; the compiler pads it with wait states, and once dropped them where a short uniform branch for
+    the partly filled tile sat between the two (hence that tile being a template instantiation in both kernels, and the explicit
+    wait states before the epilogue's first read of the accumulators).  The symptom was wrong scores of the last tile only.  Here the
+    last tile is partly filled (S % 16 = rest) and carries nearly all of the softmax weight, through both block shapes (<= 256
+    blocks: eight waves, above: four) and both kernels, against an elementwise bound."""
+    from common import attention_error_bound
+    dev = require_gpu()
+    from gaac_amd import attention, Codec, TileEncoder
+    from gaac_amd.kernel import bf16_attention
+    n_kv, G, S = 8, 4, 16 * 40 + rest
+    assert (B * n_kv * nsplit <= 256) == (B == 1)
+    rng = np.random.default_rng(100 + rest)
+    u = rng.standard_normal((B, n_kv, 1, 128)).astype(np.float32)
+    q16 = O.f32_to_bf16_rne((u + 0.3 * rng.standard_normal((B, n_kv, G, 128)).astype(np.float32)).reshape(B, n_kv * G, 128))
+    kf = rng.standard_normal((B * n_kv, S, 128)).astype(np.float32)
+    kf[:, S - rest:] = 1.0 * u.reshape(B * n_kv, 1, 128) + 0.05 * kf[:, S - rest:]
+    k16, v16 = O.f32_to_bf16_rne(kf), _soft16(B * n_kv, S, seed=200 + rest)
+    k, v, q = to_bf16(k16, dev), to_bf16(v16, dev), to_bf16(q16, dev)
+    if kernel == "compressed":
+        kp, vp = TileEncoder("k").encode(Codec(n_kv).calibrate(k), k), TileEncoder("v").encode(Codec(n_kv).calibrate(v), v)
+        out = attention(q, kp, vp, SCALE, nsplit=nsplit)
+    else:
+        out = bf16_attention(q, k, v, SCALE, nsplit=nsplit)
+    got = O.bf16_to_f32(to_u16(out))
+    for b in range(B):
+        kb = k16[b * n_kv:(b + 1) * n_kv].transpose(1, 0, 2); vb = v16[b * n_kv:(b + 1) * n_kv].transpose(1, 0, 2)
+        ref, tol = attention_error_bound(q16[b], kb, vb, SCALE)
+        # the case is what it claims: more than half of the weight sits in the last `rest` tokens
+        s = (O.bf16_to_f32(q16[b, :G]).astype(np.float64) @ O.bf16_to_f32(kb[:, 0]).astype(np.float64).T) * SCALE
+        p = np.exp(s - s.max(-1, keepdims=True)); p /= p.sum(-1, keepdims=True)
+        assert p[:, S - rest:].sum(-1).min() > 0.5
+        assert (np.abs(got[b] - ref) <= tol).all(), (kernel, B, nsplit, rest, b, np.abs(got[b] - ref).max())
+
+
 def test_random_shapes_lengths_and_split_counts():
     """Seeded sweep over ragged lengths (partly filled last tile, fewer tiles than waves or splits), group sizes and split counts,
     through both block shapes (launches above 256 blocks use four-wave blocks)."""

@@ -128,7 +128,7 @@ def test_overflow_is_flagged_not_written():
     cache.growable = False
     big = to_bf16(np.full((1, N_KV, 128), 0x7F00, dtype=np.uint16), dev)
     for i in range(16): cache.append(slots, big, big)
-    with pytest.raises(RuntimeError, match="escape stream"):
+    with pytest.raises(RuntimeError, match="escape window"):
         cache.check_capacity()
     assert int(cache.k.ovf_used.max()) == 0 and int(cache.k.flags.abs().max()) == 0
 
