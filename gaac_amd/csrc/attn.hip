@@ -65,9 +65,10 @@ __device__ __forceinline__ u32 pack_bf16x2(float lo, float hi) {
 // (batch row, kv head), without atomics and without any block waiting for a store acknowledgement on its way out:
 //
 //   * One word, *epoch, holds the epoch of the last merged launch.  Every block reads it while its first tiles are in flight; this
-//     launch's EPOCH is that value + 1, the same for all blocks (only the last block of the grid writes the word, as its very last
-//     action; it is the last to start, so every block has read the word long before).  Records of any earlier launch, whatever its
-//     shape, carry a smaller epoch.
+//     launch's EPOCH is that value + 1 (skipping 0 when the 32-bit counter wraps), the same for all blocks (only the last block of
+//     the grid writes the word, as its very last action; it is the last to start, so every block has read the word long before).
+//     A record slot read by a launch was last written by an earlier launch, whatever its shape, under another epoch (the same
+//     value returns only after 2^32 - 1 launches on the same records), or never, and then holds the unused epoch 0.
 //   * A partial value travels as one 64-bit record (fp32 bits | epoch << 32) written with a single 64-bit store: a reader sees either
 //     the whole record of this launch or an older one, never a torn one (naturally aligned 64-bit accesses are single-copy atomic),
 //     so no fence, flag or acknowledgement orders data against a separate signal.  Records are written with agent-scope stores
@@ -92,7 +93,8 @@ constexpr int MERGE_SPIN_LIMIT = 1 << 16;      // re-reads of a chunk before the
 // (no branch around the load: a load under a branch is waited for where the branch ends, together with everything issued before it)
 __device__ __forceinline__ u32 load_epoch(const AttnArgs& A, int bh) {
   const u32* p = A.epochs ? A.epochs : reinterpret_cast<const u32*>(A.q);
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;
+  const u32 e = __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return e + 1u + (e == 0xFFFFFFFFu ? 1u : 0u);      // epoch 0 is never used: zeroed records stay stale when the counter wraps
 }
 // A block barrier that orders LDS traffic only.  (__syncthreads() also waits for the block's global stores to be acknowledged,
 // which for write-through stores is a trip to memory.)

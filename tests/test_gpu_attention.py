@@ -92,6 +92,25 @@ def test_fused_merge_equals_the_two_kernel_launch_on_a_reused_workspace():
         assert int(ws.epoch) == (1 if ns > 1 else 0)
 
 
+def test_epoch_counter_wraps_past_zero():
+    """The epoch is a 32-bit counter; 0 is what zeroed (never written) records carry, so the launch after epoch 0xFFFFFFFF takes 1."""
+    dev = require_gpu()
+    from gaac_amd.kernel import attn_launch, AttnWorkspace
+    B, n_kv, G, S, ns = 1, 4, 4, 2048, 12
+    _, _, kp, vp = _pages(B, n_kv, S, dev, seed=41)
+    n_q = n_kv * G
+    q = to_bf16(randn_bf16((B * n_q, 128), seed=9, scale=0.3), dev)
+    SL = torch.full((B * n_kv,), S, dtype=torch.int32, device=dev)
+    ws = AttnWorkspace(B * n_q, ns, torch.bfloat16, dev)
+    run = lambda ph: attn_launch(kp, vp, q, None, n_q, n_kv, SL, kp.sm.shape[1] // 128, SCALE, ns, ws=ws, phase=ph, S_all=S).float().clone()
+    two = run("both")
+    ws.reset()
+    ws.epoch.fill_(-3)      # 0xFFFFFFFD
+    for want in (-2, -1, 1, 2):
+        assert (run("fused") - two).abs().max().item() <= 2.0 ** -7 * two.abs().max().item()
+        assert int(ws.epoch) == want
+
+
 def test_launch_shapes_that_share_a_workspace_do_not_mix_their_records():
     """attention() without a workspace uses one shared per (rows, splits): (1, 8, 4) and (1, 2, 16) at 4096 tokens have the same 32 rows
     and 16 splits but other kv heads, so each launch finds the other shape's records in the buffers.  The epoch is one word per
