@@ -116,12 +116,13 @@ __device__ __forceinline__ void merge_half_head(const AttnArgs& A, long row, int
   float* fs = X.f[wave]; float* ls = X.l[wave];
   constexpr int CH = 8;      // one round for up to 8 NW splits
   bool ok = true;
-  // all loads of the first round are issued before the first use: the wave's first CH accumulator rows ...
+  // all loads of the first round are issued before the first use, none under a branch (a slot past the end reads the last slot
+  // instead and is ignored): the wave's first CH accumulator rows ...
   u64 v[CH];
 #pragma unroll
-  for (int k = 0; k < CH; ++k) { const int s = wave + NW * k; v[k] = s < nslot ? ll_load(ra + (long)s * D) : 0ull; }
+  for (int k = 0; k < CH; ++k) v[k] = ll_load(ra + (long)min(wave + NW * k, nslot - 1) * D);
   // ... then m / l of slots 0..63 (one slot per lane); everything is re-read together until it carries this launch's epoch
-  u64 mr = lane < nslot ? ll_load(rm + lane) : 0ull, lr = lane < nslot ? ll_load(rl + lane) : 0ull;
+  u64 mr = ll_load(rm + min(lane, nslot - 1)), lr = ll_load(rl + min(lane, nslot - 1));
   GAAC_MSTAMP(0, wall_clock64());
   for (int spin = 0;; ++spin) {
     bool stale = lane < nslot && (ll_stale(mr, epoch) || ll_stale(lr, epoch));
@@ -200,7 +201,11 @@ __device__ __forceinline__ int merge_ranks(int G, int nslot) { return min(min(16
 template <int NW>
 __device__ __forceinline__ void merge_heads(const AttnArgs& A, long qh0, int G, u32 epoch, int rank, int mergers, int tid, MergeScratch<NW>& X) {
   const int wave = tid >> 6, lane = tid & 63;
-  for (int item = rank; item < 2 * G; item += mergers) merge_half_head<NW>(A, qh0 + (item >> 1), item & 1, epoch, X, wave, lane);
+  // The first item stands outside the loop: at a loop header the compiler waits for every memory operation in flight, which here
+  // would be the acknowledgement of the block's own record stores (a round trip to memory) before the first record load is issued.
+  int item = rank;
+  if (item < 2 * G) { merge_half_head<NW>(A, qh0 + (item >> 1), item & 1, epoch, X, wave, lane); item += mergers; }
+  for (; item < 2 * G; item += mergers) merge_half_head<NW>(A, qh0 + (item >> 1), item & 1, epoch, X, wave, lane);
   // the last block of the grid advances the epoch word for the next launch (the blocks of this launch have read it long ago: they
   // all started before this block did)
   if (blockIdx.x == gridDim.x - 1 && tid == 0) __hip_atomic_store(A.epochs, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -877,20 +882,26 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
 #pragma unroll
       for (int r = 0; r < 4; ++r) M.acc[wave][a][chan_v(8 * (4 * q + r) + i)] = acc[i][r];
   }
+  GAAC_MSTAMP(5, wall_clock64());
   __syncthreads();
+  GAAC_MSTAMP(6, wall_clock64());
   const bool fused = A.epochs != nullptr;
   const int mergers = merge_ranks(G, A.nslot), rank = (int)blockIdx.x % A.nsplit - (A.nsplit - mergers);      // the head's last blocks to start
   const int d = tid & 127;
   for (int g = tid >> 7; g < G; g += NT / 128) {
+    // every LDS read up front and none under a branch: nine dependent round trips otherwise
+    float mv[NW + 1], lv[NW + 1], av[NW + 1];
+#pragma unroll
+    for (int w = 0; w < NW + 1; ++w) { mv[w] = M.m[w][g]; lv[w] = M.l[w][g]; av[w] = M.acc[w][g][d]; }
     float Mx = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < NW + 1; ++w) Mx = fmaxf(Mx, M.m[w][g]);
+    for (int w = 0; w < NW + 1; ++w) Mx = fmaxf(Mx, mv[w]);
     float Lc = 0.f, Ac = 0.f;
 #pragma unroll
     for (int w = 0; w < NW + 1; ++w) {
-      const bool live = M.m[w][g] != -INFINITY;          // an empty partial's accumulator may hold anything
-      const float f = live ? __builtin_amdgcn_exp2f(M.m[w][g] - Mx) : 0.f;
-      Lc += M.l[w][g] * f; Ac += live ? M.acc[w][g][d] * f : 0.f;
+      const bool live = mv[w] != -INFINITY;          // an empty partial's accumulator may hold anything
+      const float f = live ? __builtin_amdgcn_exp2f(mv[w] - Mx) : 0.f;
+      Lc += lv[w] * f; Ac += (live ? av[w] : 0.f) * f;
     }
     const long pidx = (qh0 + g) * A.nslot + split;
     if (!fused) {
