@@ -567,13 +567,21 @@ __device__ __forceinline__ void unit_x_words(const KindRegs& R, const AttnLds& L
 
 // PARTIAL: the tile is the last one of the sequence and only partly filled (rows >= S are masked out).  It is a template
 // parameter, not a run-time branch, so that no branch separates the score MFMAs from the first read of their result.
-template <bool PAGED, bool PARTIAL, bool SLOW>
-__device__ __forceinline__ void consume_tile(const TileRegs& R, WaveState& st, const AttnLds& L, const Bases& B,
-                                             u32 kto, u32 vto, int tile, int S, float scale_log2e, int a, int q,
-                                             const u32x4 (&qf)[4]) {
+template <bool PAGED, bool PARTIAL>
+__device__ __forceinline__ void consume(const TileRegs& R, WaveState& st, const AttnLds& L, const Bases& B,
+                                        u32 kto, u32 vto, int tile, int S, float scale_log2e, int a, int q,
+                                        const u32x4 (&qf)[4]) {
+  // A tile needs the SLOW look-up of its escape words when some lane holds two or more raw groups (about 1 tile in 100 at 0.3 % raw
+  // groups).  The choice is one wave-uniform branch around the look-ups only, ahead of all the matrix products of the tile.
   u32x4 xk[4], xv[4], bk[4], bv[4];
-  unit_x_words<KIND_K, SLOW>(R.k, L, esc_of_tile<PAGED>(B.kov, kto, B.TS), a, q, xk, bk);
-  unit_x_words<KIND_V, SLOW>(R.v, L, esc_of_tile<PAGED>(B.vov, vto, B.TS), a, q, xv, bv);
+  const u32 kr = __builtin_amdgcn_ubfe(R.k.f, 8 * q, 8) & 0xAAu, vr = __builtin_amdgcn_ubfe(R.v.f, 8 * q, 8) & 0xAAu;
+  if (__builtin_expect(__builtin_amdgcn_ballot_w64(((kr & (kr - 1u)) | (vr & (vr - 1u))) != 0u) != 0, 0)) {
+    unit_x_words<KIND_K, true>(R.k, L, esc_of_tile<PAGED>(B.kov, kto, B.TS), a, q, xk, bk);
+    unit_x_words<KIND_V, true>(R.v, L, esc_of_tile<PAGED>(B.vov, vto, B.TS), a, q, xv, bv);
+  } else {
+    unit_x_words<KIND_K, false>(R.k, L, esc_of_tile<PAGED>(B.kov, kto, B.TS), a, q, xk, bk);
+    unit_x_words<KIND_V, false>(R.v, L, esc_of_tile<PAGED>(B.vov, vto, B.TS), a, q, xv, bv);
+  }
   // ---- scores: S[tok 4q+r][head a]
   f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -626,17 +634,6 @@ __device__ __forceinline__ void consume_tile(const TileRegs& R, WaveState& st, c
     st.acc[pp] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, lo), pb, st.acc[pp], 0, 0, 0);
     st.acc[pp + 4] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4, hi), pb, st.acc[pp + 4], 0, 0, 0);
   }
-}
-
-// A tile needs the SLOW instantiation when some lane holds two or more raw groups (about 1 tile in 100 at 0.3 % raw groups).
-template <bool PAGED, bool PARTIAL>
-__device__ __forceinline__ void consume(const TileRegs& R, WaveState& st, const AttnLds& L, const Bases& B, u32 kto, u32 vto, int tile,
-                                        int S, float scale_log2e, int a, int q, const u32x4 (&qf)[4]) {
-  const u32 kr = __builtin_amdgcn_ubfe(R.k.f, 8 * q, 8) & 0xAAu, vr = __builtin_amdgcn_ubfe(R.v.f, 8 * q, 8) & 0xAAu;
-  if (__builtin_expect(__builtin_amdgcn_ballot_w64(((kr & (kr - 1u)) | (vr & (vr - 1u))) != 0u) != 0, 0))
-    consume_tile<PAGED, PARTIAL, true>(R, st, L, B, kto, vto, tile, S, scale_log2e, a, q, qf);
-  else
-    consume_tile<PAGED, PARTIAL, false>(R, st, L, B, kto, vto, tile, S, scale_log2e, a, q, qf);
 }
 
 // Next tile for a wave from the block's counter in LDS (lane 0's value counts).  The caller makes it uniform only when it needs it,
