@@ -217,3 +217,61 @@ def test_config_3_paged_pool_at_full_size():
         sk = torch.empty(cur[i], n_kv, D, dtype=torch.bfloat16, device=dev); sv = torch.empty_like(sk)
         st.decode_blocks(buf, pairs, sk, sv)
         assert torch.equal(sk.view(torch.int16), hist_k[i].view(torch.int16)) and torch.equal(sv.view(torch.int16), hist_v[i].view(torch.int16))
+
+
+def test_config_4_call_site_at_full_size():
+    """Config 4: the Llama-3-8B architecture (32 layers, hidden 4096, 32 q / 8 kv heads, FFN 14336, vocab 128256; random bf16 weights),
+    batch 4 at 32768-token contexts, through the engine-shaped call site.  Teacher forcing makes the compressed and the uncompressed
+    run comparable step by step: after the prefill and after 6 forced decode steps every layer's cache holds the same K/V bits in
+    both runs where their inputs are the same (all layers during prefill, layer 0 throughout; position-weighted checksums), the
+    rows a layer appended are bit for bit what it was handed, and the logits of every step differ by no more than a small multiple
+    of what the uncompressed run itself changes by when only its split count (summation order) changes."""
+    dev = require_gpu()
+    from gaac_amd.serving import ModelConfig, Weights, DecodeRunner
+    B, ctx, steps = 4, 32768, 6
+    cfg = ModelConfig(max_len=ctx + 64)
+    w = Weights(cfg, dev, seed=0)
+    g = torch.Generator(device=dev).manual_seed(1)
+    prompts = [torch.randint(0, cfg.vocab, (ctx,), generator=g, device=dev) for _ in range(B)]
+    forced = torch.randint(0, cfg.vocab, (steps, B), generator=g, device=dev)
+
+    def checksum(x, L):
+        bits = x[:L].contiguous().view(torch.int16).to(torch.int64).flatten()
+        return int((bits * (torch.arange(bits.numel(), device=dev) % 65521 + 1)).sum().item())
+
+    def run(kv, nsplit=None, sums=True):
+        r = DecodeRunner(w, n_slots=B, kv=kv)
+        first = torch.stack([r.prefill(i, p).argmax() for i, p in enumerate(prompts)])
+        fed = [[] for _ in range(cfg.n_layers)]
+        hooks = [at.register_forward_hook(lambda m, args, out, l=l: fed[l].append((args[1].clone(), args[2].clone()))) for l, at in enumerate(r.attn)]
+        r.start_decode(first, use_graph=False, nsplit=nsplit)
+        _, lg = r.decode(steps, forced=forced, keep_logits=True)
+        for h in hooks: h.remove()
+        cs = []
+        for l in range(cfg.n_layers if sums else 0):
+            for slot in range(B):
+                L = ctx + steps if l == 0 else ctx
+                if kv == "gaac":
+                    dk, dv = r.caches[l].decompress(slot)
+                    assert dk.shape[0] == ctx + steps
+                    nk = torch.stack([f[0][slot] for f in fed[l]]); nv = torch.stack([f[1][slot] for f in fed[l]])
+                    assert torch.equal(dk[ctx:].view(torch.int16), nk.view(torch.int16)) and torch.equal(dv[ctx:].view(torch.int16), nv.view(torch.int16)), (l, slot)
+                else:
+                    c, h0 = r.caches[l], slot * cfg.n_kv_heads
+                    dk, dv = c.k[h0:h0 + cfg.n_kv_heads, :L].transpose(0, 1), c.v[h0:h0 + cfg.n_kv_heads, :L].transpose(0, 1)
+                cs.append((checksum(dk, L), checksum(dv, L)))
+                del dk, dv
+        st = r.kv_stats()
+        del r
+        torch.cuda.empty_cache()
+        return first, lg, cs, st
+
+    first_g, lg, cs_g, st_g = run("gaac")
+    first_b, lb, cs_b, _ = run("bf16")
+    assert torch.equal(first_g, first_b)
+    assert cs_g == cs_b
+    _, ln, _, _ = run("bf16", nsplit=5, sums=False)
+    d = (lg - lb).abs().flatten(1); dn = (ln - lb).abs().flatten(1)
+    for i in range(steps):
+        assert d[i].max().item() <= 4 * dn.max().item() and d[i].mean().item() <= 2 * dn.mean().item(), (i, d[i].max().item(), dn.max().item())
+    assert st_g["tokens"] == B * (ctx + steps) and 1.3 < st_g["ratio"] < 1.5
