@@ -413,8 +413,8 @@ __device__ __forceinline__ void tables_store(AttnLds& L, TableRegs Tr, int tid, 
 // ---------------------------------------------------------------------------------------------------- tile loaders
 struct KindRegs {                // one lane's view of one tile (K or V)
   Payload pay;
-  u32 f;                         // tag word of the lane's line
-  u32 pos0;                      // offset of the lane's first unit in the tile's escape bytes
+  u32 f;                         // the lane's four tags (bits 8q .. 8q+7 of the tag word of its line)
+  u32 pos0;                      // offset of the lane's first unit's escape bytes: in the head's stream | in the tile (paged)
   u32x2 e;                       // the 8 escape bytes from pos0 on
 };
 struct TileRegs { KindRegs k, v; };
@@ -480,15 +480,18 @@ __device__ __forceinline__ void load_tile_escapes(const Bases& B, int lane, cons
   // escape bytes per line of K (low half) and V (high half): one scan for both
   const u32 rb = (u32)esc_bytes(Tg.kfl) | ((u32)esc_bytes(Tg.vfl) << 16);
   const u32 excl = row_scan16(rb) - rb;
-  R.k.f = Tg.kfl; R.v.f = Tg.vfl;
+  // What the consumer needs of the tag words and tile offsets is computed here, into registers of the tile: the tag registers are
+  // then free for the next tags, and nothing has to be copied out of a register that a load is still writing.
+  R.k.f = __builtin_amdgcn_ubfe(Tg.kfl, 8 * q, 8); R.v.f = __builtin_amdgcn_ubfe(Tg.vfl, 8 * q, 8);
   R.k.pos0 = (excl & 0xFFFFu) + (u32)esc_prefix(Tg.kfl, 8 * q);
   R.v.pos0 = (excl >> 16) + (u32)esc_prefix(Tg.vfl, 8 * q);
   if (PAGED) {
     R.k.e = load_u32x2_unaligned(esc_of_tile<PAGED>(B.kov, __builtin_amdgcn_readfirstlane(Tg.kto), B.TS) + R.k.pos0);
     R.v.e = load_u32x2_unaligned(esc_of_tile<PAGED>(B.vov, __builtin_amdgcn_readfirstlane(Tg.vto), B.TS) + R.v.pos0);
   } else {      // stream base (uniform) + 32-bit offset (tile offset + position in the tile)
-    R.k.e = load_u32x2_unaligned(B.kov + (u32)(Tg.kto + R.k.pos0));
-    R.v.e = load_u32x2_unaligned(B.vov + (u32)(Tg.vto + R.v.pos0));
+    R.k.pos0 += Tg.kto; R.v.pos0 += Tg.vto;
+    R.k.e = load_u32x2_unaligned(B.kov + R.k.pos0);
+    R.v.e = load_u32x2_unaligned(B.vov + R.v.pos0);
   }
 }
 template <bool PAGED>
@@ -533,7 +536,7 @@ __device__ __forceinline__ u32x4 raw_x_words(u32 lo, u32 hi, const u32x4& b4w) {
 template <int KIND, bool SLOW>
 __device__ __forceinline__ void unit_x_words(const KindRegs& R, const AttnLds& L, const uint8_t* __restrict__ esc_tile, int a, int q,
                                              u32x4* __restrict__ x, u32x4* __restrict__ bw) {
-  const u32 tag8 = __builtin_amdgcn_ubfe(R.f, 8 * q, 8);
+  const u32 tag8 = R.f;
   const u32 eb4 = __builtin_amdgcn_perm(R.e[1], R.e[0], L.sel[tag8]);
   const u32x4* tab = KIND == KIND_K ? &L.bwk[0][4 * q] : &L.bwv[0][a];      // row of unit 0 at tier 0; tier 1 is NG rows further
 #pragma unroll
@@ -557,7 +560,12 @@ __device__ __forceinline__ void unit_x_words(const KindRegs& R, const AttnLds& L
         const u32 t = (tag8 >> (2 * u)) & 3u;
         if (t) {
           const u64 v = load_u64_unaligned(esc_tile + R.pos0 + off);
-          x[u] = t == 1u ? L.xlut[(u32)v & 0xFFu] : raw_x_words((u32)v, (u32)(v >> 32), bw[u]);
+          // The loaded bytes are waited for here, in the block that issues the load: their two users below sit in separate divergent
+          // blocks, and a load that is still pending on the path past both makes the compiler wait for every load in flight wherever
+          // its register is reused, on the common path as well.
+          u32 vlo = (u32)v, vhi = (u32)(v >> 32);
+          asm volatile("" : "+v"(vlo), "+v"(vhi));
+          x[u] = t == 1u ? L.xlut[vlo & 0xFFu] : raw_x_words(vlo, vhi, bw[u]);
         }
         off += (u32)tag_size(t);
       }
@@ -574,13 +582,13 @@ __device__ __forceinline__ void consume(const TileRegs& R, WaveState& st, const 
   // A tile needs the SLOW look-up of its escape words when some lane holds two or more raw groups (about 1 tile in 100 at 0.3 % raw
   // groups).  The choice is one wave-uniform branch around the look-ups only, ahead of all the matrix products of the tile.
   u32x4 xk[4], xv[4], bk[4], bv[4];
-  const u32 kr = __builtin_amdgcn_ubfe(R.k.f, 8 * q, 8) & 0xAAu, vr = __builtin_amdgcn_ubfe(R.v.f, 8 * q, 8) & 0xAAu;
+  const u32 kr = R.k.f & 0xAAu, vr = R.v.f & 0xAAu;
   if (__builtin_expect(__builtin_amdgcn_ballot_w64(((kr & (kr - 1u)) | (vr & (vr - 1u))) != 0u) != 0, 0)) {
-    unit_x_words<KIND_K, true>(R.k, L, esc_of_tile<PAGED>(B.kov, kto, B.TS), a, q, xk, bk);
-    unit_x_words<KIND_V, true>(R.v, L, esc_of_tile<PAGED>(B.vov, vto, B.TS), a, q, xv, bv);
+    unit_x_words<KIND_K, true>(R.k, L, PAGED ? esc_of_tile<PAGED>(B.kov, kto, B.TS) : B.kov, a, q, xk, bk);
+    unit_x_words<KIND_V, true>(R.v, L, PAGED ? esc_of_tile<PAGED>(B.vov, vto, B.TS) : B.vov, a, q, xv, bv);
   } else {
-    unit_x_words<KIND_K, false>(R.k, L, esc_of_tile<PAGED>(B.kov, kto, B.TS), a, q, xk, bk);
-    unit_x_words<KIND_V, false>(R.v, L, esc_of_tile<PAGED>(B.vov, vto, B.TS), a, q, xv, bv);
+    unit_x_words<KIND_K, false>(R.k, L, nullptr, a, q, xk, bk);
+    unit_x_words<KIND_V, false>(R.v, L, nullptr, a, q, xv, bv);
   }
   // ---- scores: S[tok 4q+r][head a]
   f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
@@ -756,7 +764,10 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
 #define TILE(i) (tlo + (i))
   int iA = wave, iB = wave + NW;
   TileRegs R0, R1;
-  TagRegs Tg, TgC0, TgC1;
+  // Two sets of tag registers, used in turn: a set is loaded one tile before the payload that needs it, read where that payload's
+  // escape bytes are fetched, and then free.  (Paged pool: slot indices and the raw mark of the tile in R0 / R1, scalar values.)
+  TagRegs Tg, TgB;
+  struct TileMeta { u32 kto, vto; int raw; } m0 = {0u, 0u, 0}, m1 = {0u, 0u, 0};
   const bool any_tile = iA < n_own;
   // The wave's first tile: tag words and payload.  Without a branch where the addresses are always valid (a wave without tiles reads
   // a tile it does not consume): behind a branch the compiler can no longer count the loads in flight and turns every later wait
@@ -799,26 +810,26 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
 
   if (!PAGED) { B.kov = A.k.ovf + __builtin_amdgcn_readfirstlane((int)khs); B.vov = A.v.ovf + __builtin_amdgcn_readfirstlane((int)vhs); }
   if (any_tile) {
-    TgC0 = Tg;
+    if (PAGED) m0 = TileMeta{Tg.kto, Tg.vto, Tg.raw};
     load_tile_escapes<PAGED>(B, lane, Tg, R0);
-    load_tags<PAGED>(B, TT, TILE(min(iB, icl)), a, Tg);
+    load_tags<PAGED>(B, TT, TILE(min(iB, icl)), a, TgB);
     int vC = take_tile(&next_tile, n_own, lane);
     // The loop is entered with the loads in flight in the same order as on its back edge (tile, then the next tile's tags), so the
     // waits inside it stay waits for exactly the loads they need.
-    while (true) {        // R0 = tile iA, Tg = tags of tile iB
-      TgC1 = Tg;
-      load_tile<PAGED>(B, TILE(min(iB, icl)), lane, Tg, R1);
+    while (true) {        // R0 = tile iA, TgB = tags of tile iB
+      if (PAGED) m1 = TileMeta{TgB.kto, TgB.vto, TgB.raw};
+      load_tile<PAGED>(B, TILE(min(iB, icl)), lane, TgB, R1);
       const int vD = take_tile(&next_tile, n_own, lane);
       const int iC = uniform_tile(vC);
       load_tags<PAGED>(B, TT, TILE(min(iC, icl)), a, Tg);
-      if (!PAGED || !TgC0.raw) consume<PAGED, false>(R0, st, L, B, TgC0.kto, TgC0.vto, TILE(iA), S, A.scale_log2e, a, q, qf);
+      if (!PAGED || !m0.raw) consume<PAGED, false>(R0, st, L, B, m0.kto, m0.vto, TILE(iA), S, A.scale_log2e, a, q, qf);
       if (iB >= n_own) break;
-      TgC0 = Tg;
+      if (PAGED) m0 = TileMeta{Tg.kto, Tg.vto, Tg.raw};
       load_tile<PAGED>(B, TILE(min(iC, icl)), lane, Tg, R0);
       const int vE = take_tile(&next_tile, n_own, lane);
       const int iD = uniform_tile(vD);
-      load_tags<PAGED>(B, TT, TILE(min(iD, icl)), a, Tg);
-      if (!PAGED || !TgC1.raw) consume<PAGED, false>(R1, st, L, B, TgC1.kto, TgC1.vto, TILE(iB), S, A.scale_log2e, a, q, qf);
+      load_tags<PAGED>(B, TT, TILE(min(iD, icl)), a, TgB);
+      if (!PAGED || !m1.raw) consume<PAGED, false>(R1, st, L, B, m1.kto, m1.vto, TILE(iB), S, A.scale_log2e, a, q, qf);
       if (iC >= n_own) break;
       iA = iC; iB = iD; vC = vE;
     }
