@@ -100,46 +100,48 @@ __device__ __forceinline__ u32 load_epoch(const AttnArgs& A, int bh) {
 // which for write-through stores is a trip to memory.)
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-// LDS of a merging block: per wave the (m, then factor) and l of every slot; the waves' partial sums and their verdicts.
-template <int NW> struct MergeScratch { float f[NW][MAX_SLOTS], l[NW][MAX_SLOTS]; float part[NW][64]; int ok[NW]; };
+// LDS of a merging block: per wave the (m, then weight) and l of every slot.
+template <int NW> struct MergeScratch { float f[NW][MAX_SLOTS], l[NW][MAX_SLOTS]; };
 
-// One merger's work for half a query head (64 output dims, one per lane), shared by the NW waves of the block: every wave reads the
-// m / l records of all slots (lane = slot) and the accumulator records of slots wave, wave + NW, ...; the waves' sums meet in LDS.
-// The code is kept short on purpose: it runs once per launch on a cold instruction cache, where straight-line code costs a trip to
-// the L2 per cache line.  Called by all threads of the block.
+// One merger's work for half a query head (64 output channels), shared by the NW waves of the block.  A wave owns 64 / NW channels
+// and sums them over ALL slots, so the waves exchange nothing and no block barrier lies between the records' arrival and the
+// output: lane (g, c) = (lane / CPW, lane % CPW) reads the accumulator records of channel c of the wave for the slots g, g + SG, ...
+// (SG = 64 / CPW slot groups); the groups' sums meet through DPP.  Every wave reads the m / l records of all slots (lane = slot)
+// and derives the slots' weights itself.  Called by all threads of the block.
 template <int NW>
 __device__ __forceinline__ void merge_half_head(const AttnArgs& A, long row, int half, u32 epoch, MergeScratch<NW>& X, int wave, int lane) {
-  const int nslot = A.nslot, d = 64 * half + lane;
+  constexpr int CPW = 64 / NW, SG = 64 / CPW;      // channels per wave (8 | 16), slot groups (8 | 4)
+  constexpr int CH = 8;                             // accumulator records in flight per lane: one round for up to CH * SG splits
+  const int nslot = A.nslot, g = lane / CPW, d = 64 * half + CPW * wave + lane % CPW;
   const u64* rm = reinterpret_cast<const u64*>(A.pm) + row * nslot;
   const u64* rl = reinterpret_cast<const u64*>(A.pl) + row * nslot;
   const u64* ra = reinterpret_cast<const u64*>(A.pa) + row * nslot * D + d;
   float* fs = X.f[wave]; float* ls = X.l[wave];
-  constexpr int CH = 8;      // one round for up to 8 NW splits
   bool ok = true;
   // all loads of the first round are issued before the first use, none under a branch (a slot past the end reads the last slot
-  // instead and is ignored): the wave's first CH accumulator rows ...
+  // instead and is ignored): the lane's first CH accumulator records ...
   u64 v[CH];
 #pragma unroll
-  for (int k = 0; k < CH; ++k) v[k] = ll_load(ra + (long)min(wave + NW * k, nslot - 1) * D);
+  for (int k = 0; k < CH; ++k) v[k] = ll_load(ra + (long)min(g + SG * k, nslot - 1) * D);
   // ... then m / l of slots 0..63 (one slot per lane); everything is re-read together until it carries this launch's epoch
   u64 mr = ll_load(rm + min(lane, nslot - 1)), lr = ll_load(rl + min(lane, nslot - 1));
   GAAC_MSTAMP(0, wall_clock64());
   for (int spin = 0;; ++spin) {
     bool stale = lane < nslot && (ll_stale(mr, epoch) || ll_stale(lr, epoch));
 #pragma unroll
-    for (int k = 0; k < CH; ++k) stale |= wave + NW * k < nslot && ll_stale(v[k], epoch);
+    for (int k = 0; k < CH; ++k) stale |= g + SG * k < nslot && ll_stale(v[k], epoch);
     if (__builtin_amdgcn_ballot_w64(stale) == 0) break;
     if (spin >= MERGE_SPIN_LIMIT) { ok = false; break; }
     __builtin_amdgcn_s_sleep(1);
     if (lane < nslot && ll_stale(mr, epoch)) mr = ll_load(rm + lane);
     if (lane < nslot && ll_stale(lr, epoch)) lr = ll_load(rl + lane);
 #pragma unroll
-    for (int k = 0; k < CH; ++k) { const int s = wave + NW * k; if (s < nslot && ll_stale(v[k], epoch)) v[k] = ll_load(ra + (long)s * D); }
+    for (int k = 0; k < CH; ++k) { const int s = g + SG * k; if (s < nslot && ll_stale(v[k], epoch)) v[k] = ll_load(ra + (long)s * D); }
   }
   GAAC_MSTAMP(1, wall_clock64());
-  float m = lane < nslot ? ll_value(mr) : -INFINITY;
-  if (lane < nslot) { fs[lane] = m; ls[lane] = ll_value(lr); }
-  for (int s0 = 64; ok && s0 < nslot; s0 += 64) {      // more than 64 splits: the other m / l records
+  const float m_own = lane < nslot ? ll_value(mr) : -INFINITY, l_own = lane < nslot ? ll_value(lr) : 0.f;      // slot = lane
+  float m = m_own;
+  for (int s0 = 64; ok && s0 < nslot; s0 += 64) {      // more than 64 splits: the other m / l records, kept in LDS
     const int s = s0 + lane;
     mr = s < nslot ? ll_load(rm + s) : 0ull; lr = s < nslot ? ll_load(rl + s) : 0ull;
     for (int spin = 0; __builtin_amdgcn_ballot_w64(s < nslot && (ll_stale(mr, epoch) || ll_stale(lr, epoch))) != 0; ++spin) {
@@ -150,49 +152,50 @@ __device__ __forceinline__ void merge_half_head(const AttnArgs& A, long row, int
     }
     if (s < nslot) { fs[s] = ll_value(mr); ls[s] = ll_value(lr); m = fmaxf(m, ll_value(mr)); }
   }
-  m = wave_max(m);
-  float l = 0.f;
-  for (int s = lane; s < nslot; s += 64) {      // each lane revisits the slots it wrote
-    const float pmv = fs[s], f = pmv != -INFINITY ? __builtin_amdgcn_exp2f(pmv - m) : 0.f;
+  const float mx = wave_max(m);
+  // the slots' weights go to LDS for the lanes that need them (the wave's own region: no block barrier)
+  const float f_own = m_own != -INFINITY ? __builtin_amdgcn_exp2f(m_own - mx) : 0.f;
+  float l = l_own * f_own;
+  fs[lane] = f_own;
+  for (int s = lane + 64; s < nslot; s += 64) {      // each lane revisits the slots it wrote
+    const float pmv = fs[s], f = pmv != -INFINITY ? __builtin_amdgcn_exp2f(pmv - mx) : 0.f;
     fs[s] = f; l += ls[s] * f;
   }
   l = wave_sum(l);
   wave_lds_sync();
   float acc = 0.f;
-  for (int s0 = wave; s0 < nslot; s0 += NW * CH) {
-    if (s0 != wave) {      // more than CH * NW splits: the wave's further rows
+  for (int s0 = g; s0 < nslot; s0 += SG * CH) {
+    if (s0 != g) {      // more than CH * SG splits: the lane's further records
 #pragma unroll
-      for (int k = 0; k < CH; ++k) { const int s = s0 + NW * k; v[k] = s < nslot ? ll_load(ra + (long)s * D) : 0ull; }
+      for (int k = 0; k < CH; ++k) { const int s = s0 + SG * k; v[k] = s < nslot ? ll_load(ra + (long)s * D) : 0ull; }
       for (int spin = 0; ok; ++spin) {
         bool stale = false;
 #pragma unroll
-        for (int k = 0; k < CH; ++k) stale |= s0 + NW * k < nslot && ll_stale(v[k], epoch);
+        for (int k = 0; k < CH; ++k) stale |= s0 + SG * k < nslot && ll_stale(v[k], epoch);
         if (__builtin_amdgcn_ballot_w64(stale) == 0) break;
         if (spin >= MERGE_SPIN_LIMIT) { ok = false; break; }
         __builtin_amdgcn_s_sleep(1);
 #pragma unroll
-        for (int k = 0; k < CH; ++k) { const int s = s0 + NW * k; if (s < nslot && ll_stale(v[k], epoch)) v[k] = ll_load(ra + (long)s * D); }
+        for (int k = 0; k < CH; ++k) { const int s = s0 + SG * k; if (s < nslot && ll_stale(v[k], epoch)) v[k] = ll_load(ra + (long)s * D); }
       }
     }
 #pragma unroll
     for (int k = 0; k < CH; ++k) {
-      const int s = s0 + NW * k;
+      const int s = s0 + SG * k;
       if (s < nslot) { const float f = fs[s]; acc += f != 0.f ? ll_value(v[k]) * f : 0.f; }      // an empty partial's accumulator may hold anything
     }
   }
+  // the slot groups' sums of a channel sit CPW lanes apart: across the four 16-lane rows, and for CPW = 8 also 8 lanes apart in a row
+  acc = quad_rows_sum(acc);
+  if (CPW == 8) acc += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, acc), 0x128 /* row_ror:8 */, 0xF, 0xF, false));
   GAAC_MSTAMP(2, wall_clock64());
-  X.part[wave][lane] = acc;
-  if (lane == 0) X.ok[wave] = ok;
-  lds_barrier();
-  GAAC_MSTAMP(3, wall_clock64());
-  if (wave == 0) {
-#pragma unroll
-    for (int w = 1; w < NW; ++w) { acc += X.part[w][lane]; ok = ok && X.ok[w]; }
+  ok = __builtin_amdgcn_ballot_w64(!ok) == 0;
+  if (lane < CPW) {
     const float o = ok ? (l > 0.f ? acc / l : 0.f) : __builtin_nanf("");
     A.out[row * D + d] = __builtin_bit_cast(u16, (__bf16)o);
   }
   GAAC_MSTAMP(4, wall_clock64());
-  lds_barrier();      // part is free for the block's next item
+  wave_lds_sync();      // the wave's LDS region is free for its next item
 }
 // The merge of a head is shared by its last `mergers` blocks in index order (merge_ranks): the block of rank j takes the half heads
 // j, j + mergers, ..., so that no single CU has to pull all the records.  Called by all threads of a merging block after its own
