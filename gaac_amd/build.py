@@ -13,7 +13,7 @@ LIB_TIMING = os.path.join(HERE, "libgaac_hip_timing.so")      # same sources wit
 SOURCES = ["codec.hip", "attn.hip", "cache.hip", "paged.hip", "probe.hip"]
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", 
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",      # never emit packed-FP32 VALU ops
-         # atomics here are issued by one chosen lane (tile counter in LDS, merge ticket): skip the compiler's wave-wide aggregation code
+         # atomics here are issued by one chosen lane (the tile counter in LDS): skip the compiler's wave-wide aggregation code
          "-mllvm", "-amdgpu-atomic-optimizer-strategy=None",
          "-Wno-unused-command-line-argument"]
 

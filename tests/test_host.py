@@ -95,3 +95,31 @@ def test_bytes_per_slot_closed_form():
     head = cap * 128 + cap * 48 + cap * 4 + tiles * 4 + tiles * 128 + 8 + 4 + 4 + 16 * 128 * 2 + 2 * 128
     assert CompressedKVCache.bytes_per_slot(8, 65537) == 8 * (2 * head + 4 + 4)
     assert CompressedKVCache.bytes_per_slot(8, 65537, per_sequence_bases=False) == 8 * (2 * (head - 256) + 8)
+
+
+def test_engine_context_and_attention_layer_without_a_cache():
+    """The engine-shaped surface on the host (/root/reference/nanovllm/utils/context.py:5-31): the context is one module-level object
+    with the reference's fields; an attention layer without a cache refuses to run instead of falling back to anything."""
+    import dataclasses
+    import torch
+    from gaac_amd import serving
+    names = [f.name for f in dataclasses.fields(serving.Context)]
+    assert names == ["is_prefill", "cu_seqlens_q", "cu_seqlens_k", "max_seqlen_q", "max_seqlen_k", "slot_mapping", "context_lens",
+                     "block_tables", "kv_slots", "prefill_spans"]
+    serving.set_context(True, max_seqlen_q=5, prefill_spans=[(1, 0, 5)])
+    c = serving.get_context()
+    assert c.is_prefill and c.max_seqlen_q == 5 and c.prefill_spans == [(1, 0, 5)] and c.kv_slots is None
+    serving.reset_context()
+    c = serving.get_context()
+    assert not c.is_prefill and c.prefill_spans is None and c.max_seqlen_k == 0
+    layer = serving.Attention(8, 128, 128 ** -0.5, 2)
+    assert layer.gaac is None and layer.k_cache.numel() == 0
+    q = torch.zeros(1, 8, 128, dtype=torch.bfloat16); k = torch.zeros(1, 2, 128, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="no KV cache attached"):
+        layer(q, k, k)
+    with pytest.raises(AssertionError, match="head_dim"):
+        serving.Attention(8, 64, 0.125, 2)
+    # slots from a byte budget: the closed form of the cache, no device needed for the arithmetic
+    from gaac_amd.kv_cache import CompressedKVCache
+    per_slot = 4 * CompressedKVCache.bytes_per_slot(8, 4096)
+    assert min(16, (3 * per_slot + 5) // per_slot) == 3
