@@ -16,6 +16,9 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
          # atomics here are issued by one chosen lane (the tile counter in LDS): skip the compiler's wave-wide aggregation code
          "-mllvm", "-amdgpu-atomic-optimizer-strategy=None",
          "-Wno-unused-command-line-argument"]
+# per source: the attention kernels' tile loop is a long chain of dependent LDS look-ups, decode arithmetic and matrix products with
+# only two waves per SIMD to hide latencies behind; the scheduler's ILP-first strategy measured 0.3 us faster per launch on config 1
+SOURCE_FLAGS = {"attn.hip": ["-mllvm", "-amdgpu-sched-strategy=max-ilp"]}
 
 
 def build(verbose: bool = True, extra_flags: list[str] | None = None, timing: bool = False) -> str:
@@ -25,7 +28,7 @@ def build(verbose: bool = True, extra_flags: list[str] | None = None, timing: bo
     if timing: extra_flags = [*(extra_flags or []), "-DGAAC_PHASE_TIMING"]
     for src in SOURCES:
         obj = os.path.join(CSRC, src.replace(".hip", ".timing.o" if timing else ".o"))
-        cmd = [hipcc, *FLAGS, *(extra_flags or []), "-c", os.path.join(CSRC, src), "-o", obj]
+        cmd = [hipcc, *FLAGS, *SOURCE_FLAGS.get(src, []), *(extra_flags or []), "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose: print(" ".join(cmd), flush=True)
         r = subprocess.run(cmd, capture_output=True, text=True)
         err = "\n".join(l for l in r.stderr.splitlines() if "is not a recognized feature for this target" not in l)
