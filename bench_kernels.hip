@@ -1,11 +1,14 @@
-// Measurement aid: the memory side of the fused decode-attention kernel without its arithmetic.  One block per (cache head, split), eight
+// Measurement aids of bench.py, built into libgaac_bench.so (not part of the product library libgaac_hip.so).
+//
+// gaac_stream_copy: a plain copy with 16-byte accesses per lane, the known-size kernel against which the HBM traffic counters
+// (FETCH_SIZE / WRITE_SIZE) are scaled.
+//
+// gaac_read_probe: the memory side of the fused decode-attention kernel without its arithmetic.  One block per (cache head, split), eight
 // waves, every wave fetches the tiles wave, wave + 8, ... of the block's contiguous range one tile ahead of the tile it "consumes" (an
 // xor over the loaded registers), with the attention kernel's own loads: per tile and kind two 16-byte and three 4-byte loads per lane
 // (non-temporal), and, on request, the tile's tag words, its offset in the escape stream and eight escape bytes per lane.  What this
 // kernel needs for a page is what the load pattern itself costs on the part: the floor under k_attn_split for that page.
-#include "gaac_tile.h"
-#include "gaac_capi.h"
-#include "../../include/gaac_hip.h"
+#include "gaac_tile.h"      // -I gaac_amd/csrc: the tile format and the payload loads of the attention kernel
 
 namespace gaac {
 
@@ -58,18 +61,31 @@ __global__ void __launch_bounds__(512, 1) k_read_probe(ProbeView K, ProbeView V,
   if (acc == 0x9E3779B9u) sink[0] = acc;      // keeps the loads alive; practically never written
 }
 
+__global__ void __launch_bounds__(256) k_stream_copy(const u32x4* __restrict__ src, u32x4* __restrict__ dst, long n16) {
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n16; i += (long)gridDim.x * 256) dst[i] = src[i];
+}
+
 }  // namespace gaac
 
 using namespace gaac;
+
+// both return 0, -1 for rejected arguments, or the hipError_t of a failed launch
+extern "C" int gaac_stream_copy(const void* src, void* dst, long nbytes, void* stream) {
+  if (!src || !dst || nbytes <= 0 || nbytes % 16 != 0) return -1;
+  const long n16 = nbytes / 16;
+  const int blocks = (int)((n16 + 255) / 256 < 8192 ? (n16 + 255) / 256 : 8192);
+  hipLaunchKernelGGL(k_stream_copy, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (const u32x4*)src, (u32x4*)dst, n16);
+  return (int)hipGetLastError();
+}
 
 extern "C" int gaac_read_probe(
     const uint8_t* smk, const uint8_t* ck, const int* fk, const int* tok, const uint8_t* ovk, const int* ohsk,
     const uint8_t* smv, const uint8_t* cv, const int* fv, const int* tov, const uint8_t* ovv, const int* ohsv,
     int H, int S, int S_pad, int nsplit, int with_meta, unsigned int* sink, void* stream) {
-  GAAC_REQUIRE(smk && ck && fk && tok && ovk && ohsk && smv && cv && fv && tov && ovv && ohsv && sink, "gaac_read_probe: null pointer");
-  GAAC_REQUIRE(H > 0 && S > 0 && S % T == 0 && S <= S_pad && S_pad % T == 0 && nsplit >= 1, "gaac_read_probe: bad sizes H=%d S=%d S_pad=%d nsplit=%d", H, S, S_pad, nsplit);
+  if (!(smk && ck && fk && tok && ovk && ohsk && smv && cv && fv && tov && ovv && ohsv && sink)) return -1;
+  if (!(H > 0 && S > 0 && S % T == 0 && S <= S_pad && S_pad % T == 0 && nsplit >= 1)) return -1;
   const ProbeView K{smk, ck, fk, tok, ovk, ohsk}, V{smv, cv, fv, tov, ovv, ohsv};
   if (with_meta) hipLaunchKernelGGL(k_read_probe<true>, dim3(H * nsplit), dim3(512), 0, (hipStream_t)stream, K, V, S_pad, S / T, nsplit, sink);
   else hipLaunchKernelGGL(k_read_probe<false>, dim3(H * nsplit), dim3(512), 0, (hipStream_t)stream, K, V, S_pad, S / T, nsplit, sink);
-  return launch_status("gaac_read_probe");
+  return (int)hipGetLastError();
 }

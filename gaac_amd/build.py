@@ -9,8 +9,11 @@ import os, subprocess, sys, shutil
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libgaac_hip.so")
-LIB_TIMING = os.path.join(HERE, "libgaac_hip_timing.so")      # same sources with -DGAAC_PHASE_TIMING (per-block phase time stamps)
-SOURCES = ["codec.hip", "attn.hip", "cache.hip", "paged.hip", "probe.hip"]
+LIB_TIMING = os.path.join(HERE, "libgaac_hip_timing.so")      # same sources with -DGAAC_PHASE_TIMING (per-block phase time stamps); built on demand only
+SOURCES = ["codec.hip", "attn.hip", "cache.hip", "paged.hip"]
+# bench.py's measurement aids (read probe, plain copy): their own library next to bench.py, not in the product library
+BENCH_SRC = os.path.join(os.path.dirname(HERE), "bench_kernels.hip")
+BENCH_LIB = os.path.join(os.path.dirname(HERE), "libgaac_bench.so")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", 
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",      # never emit packed-FP32 VALU ops
          # atomics here are issued by one chosen lane (the tile counter in LDS): skip the compiler's wave-wide aggregation code
@@ -45,6 +48,18 @@ def build(verbose: bool = True, extra_flags: list[str] | None = None, timing: bo
     return out
 
 
+def build_bench_lib(verbose: bool = True) -> str:
+    """bench_kernels.hip -> libgaac_bench.so (beside bench.py)."""
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    cmd = [hipcc, *FLAGS, "-I", CSRC, "-shared", BENCH_SRC, "-o", BENCH_LIB]
+    if verbose: print(" ".join(cmd), flush=True)
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError("hipcc failed on bench_kernels.hip:\n" + "\n".join(l for l in r.stderr.splitlines() if "is not a recognized feature for this target" not in l))
+    return BENCH_LIB
+
+
 if __name__ == "__main__":
     print(build())
-    print(build(timing=True))
+    print(build_bench_lib())
+    if "--timing" in sys.argv: print(build(timing=True))

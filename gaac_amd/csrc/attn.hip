@@ -15,6 +15,8 @@
 //     two-launch alternative;
 //   * k_attn_split<true, .> reads the paged slot pool through block and mode tables (paged_kernel.py:42-241).
 //   Softmax runs in base 2 (scale * log2 e folded into the scores).
+#include <atomic>
+#include <mutex>
 #include "gaac_tile.h"
 #include "gaac_capi.h"
 #include "../../include/gaac_hip.h"
@@ -34,7 +36,7 @@ struct AttnArgs {
   const int* slot; const int* sl;
   int S_pad; float scale_log2e; int nsplit; int nslot; int n_kv; int n_q; int G; int NB;
   const u16* kt; const u16* vt; const int* tl; int tcap;
-  u32* epochs; u16* out;       // fused merge: the word with the epoch of the last merged launch; pm / pl / pa then hold 64-bit records
+  u32* epochs; u16* out;       // fused merge: [0] the epoch of the last merged launch, [1] failure bits, [2 + i] arrival mark of block i; pm / pl / pa then hold 64-bit records
   int S_all;                   // >= 0: every addressed cache head holds exactly S_all compressed tokens (sl is not read)
   // paged slot pool (k_attn_split<true>): sl = tokens per batch row, bt = block table [B][bt_stride], mt = mode table, pool = tile
   // slots of TS bytes, raw = side pool of BF16 tiles; physical tile = block*2*n_kv + 2*kvh + kind
@@ -50,7 +52,7 @@ struct AttnArgs {
 #define GAAC_STAMP(k) do {} while (0)
 #define GAAC_MSTAMP(k, v) do {} while (0)
 #endif
-constexpr int MAX_CHUNK = 1024;  // tiles per split whose slot lookups a block keeps in LDS (paged mode)
+constexpr int MAX_CHUNK = 1024;  // tiles whose slot lookups a block keeps in LDS at a time (paged mode); longer splits go on in further rounds
 constexpr int SLOT_CD = TILE_SM, SLOT_FL = TILE_SM + TILE_CD, SLOT_OV = SLOT_FL + 4 * T;      // byte offsets inside a tile slot
 
 __device__ __forceinline__ float bf16_bits_to_float(u32 h) { return __uint_as_float(h << 16); }
@@ -64,9 +66,12 @@ __device__ __forceinline__ u32 pack_bf16x2(float lo, float hi) {
 // Merge of the split partials (gaac_combine, /root/reference/gaac/kernel.py:281-294) inside the split kernel, by ONE block of each
 // (batch row, kv head), without atomics and without any block waiting for a store acknowledgement on its way out:
 //
-//   * One word, *epoch, holds the epoch of the last merged launch.  Every block reads it while its first tiles are in flight; this
-//     launch's EPOCH is that value + 1 (skipping 0 when the 32-bit counter wraps), the same for all blocks (only the last block of
-//     the grid writes the word, as its very last action; it is the last to start, so every block has read the word long before).
+//   * One word, epochs[0], holds the epoch of the last merged launch.  Every block reads it while its first tiles are in flight; this
+//     launch's EPOCH is that value + 1 (skipping 0 when the 32-bit counter wraps), the same for all blocks: the word is advanced by
+//     the last block of the grid, as its very last action, and only after it has SEEN the arrival mark of every block of the grid
+//     (epochs[2 + block], stored by the block once its first wave is through its tiles: a block that has marked has read the word
+//     long ago; blocks of a grid larger than the GPU holds start whenever a CU of their XCD frees up, in no order the other XCDs
+//     know of).
 //     A record slot read by a launch was last written by an earlier launch, whatever its shape, under another epoch (the same
 //     value returns only after 2^32 - 1 launches on the same records), or never, and then holds the unused epoch 0.
 //   * A partial value travels as one 64-bit record (fp32 bits | epoch << 32) written with a single 64-bit store: a reader sees either
@@ -75,12 +80,12 @@ __device__ __forceinline__ u32 pack_bf16x2(float lo, float hi) {
 //     (write-through) and read with agent-scope loads (they bypass the reader's L2): the blocks of a head sit on different XCDs.
 //   * The MERGERS are the head's last (up to sixteen) blocks in index order; each takes a share of the head's output (half a query head
 //     per wave), because one CU pulls records at only ~80 GB/s.  Once a merger has stored its own partial it loads the records of its
-//     share from all blocks of the head and re-reads those whose epoch is not yet the launch's.  Workgroups start in index order and
-//     a head's blocks are consecutive, so everything a merger waits for is running, done, or one of the at most fifteen later mergers
-//     of the same head, which get the next free CUs; blocks that are not mergers wait for nobody.  The wait is bounded all the same
-//     (MERGE_SPIN_LIMIT re-reads, then the rows are written as NaN), so that neither a damaged epoch word nor another start order
-//     can hang the GPU.
-//   * Launches that share the records and the epoch word must be ordered on one stream.  To re-arm after a failed launch, zero both.
+//     share from all blocks of the head and re-reads those whose epoch is not yet the launch's.  Everything a merger waits for is
+//     running, done, or one of the at most fifteen later mergers of the same head, which wait for nobody but each other's stores,
+//     and those precede every wait.  The wait is bounded all the same (MERGE_SPIN_LIMIT re-reads): a merger that gives up writes its
+//     rows as NaN and sets bit 0 of epochs[1]; the grid's last block sets bit 1 if it gives up waiting for the other blocks (it then
+//     leaves the epoch word alone).  The owner of the workspace polls epochs[1] and re-arms after a failure.
+//   * Launches that share the records and the epoch words must be ordered on one stream.  To re-arm after a failed launch, zero all.
 typedef __attribute__((ext_vector_type(4))) float f32x4v;
 __device__ __forceinline__ void store_partial(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
 __device__ __forceinline__ void ll_store(u64* p, float v, u32 epoch) {
@@ -108,6 +113,9 @@ template <int NW> struct MergeScratch { float f[NW][MAX_SLOTS], l[NW][MAX_SLOTS]
 // output: lane (g, c) = (lane / CPW, lane % CPW) reads the accumulator records of channel c of the wave for the slots g, g + SG, ...
 // (SG = 64 / CPW slot groups); the groups' sums meet through DPP.  Every wave reads the m / l records of all slots (lane = slot)
 // and derives the slots' weights itself.  Called by all threads of the block.
+__device__ __forceinline__ void merge_failed(const AttnArgs& A, u32 bit) {
+  __hip_atomic_fetch_or(A.epochs + 1, bit, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 template <int NW>
 __device__ __forceinline__ void merge_half_head(const AttnArgs& A, long row, int half, u32 epoch, MergeScratch<NW>& X, int wave, int lane) {
   constexpr int CPW = 64 / NW, SG = 64 / CPW;      // channels per wave (8 | 16), slot groups (8 | 4)
@@ -190,6 +198,7 @@ __device__ __forceinline__ void merge_half_head(const AttnArgs& A, long row, int
   if (CPW == 8) acc += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, acc), 0x128 /* row_ror:8 */, 0xF, 0xF, false));
   GAAC_MSTAMP(2, wall_clock64());
   ok = __builtin_amdgcn_ballot_w64(!ok) == 0;
+  if (!ok && lane == 0) merge_failed(A, 1u);
   if (lane < CPW) {
     const float o = ok ? (l > 0.f ? acc / l : 0.f) : __builtin_nanf("");
     A.out[row * D + d] = __builtin_bit_cast(u16, (__bf16)o);
@@ -201,17 +210,65 @@ __device__ __forceinline__ void merge_half_head(const AttnArgs& A, long row, int
 // j, j + mergers, ..., so that no single CU has to pull all the records.  Called by all threads of a merging block after its own
 // partial has been stored and every thread is done with the LDS that X aliases.
 __device__ __forceinline__ int merge_ranks(int G, int nslot) { return min(min(16, 2 * G), nslot); }
+// Arrival marks: epochs[2 + i] = the epoch block i of the grid works under, stored by the block's first wave when it leaves its tile
+// loop (long after it read the epoch word, well before the block publishes its partial).  The grid's last block reads all marks
+// before it advances the epoch word.
+constexpr int EPOCH_WORDS = 2;      // words of the epoch buffer ahead of the arrival marks
+__device__ __forceinline__ void mark_arrival(const AttnArgs& A, u32 epoch) {
+  __hip_atomic_store(A.epochs + EPOCH_WORDS + blockIdx.x, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 template <int NW>
 __device__ __forceinline__ void merge_heads(const AttnArgs& A, long qh0, int G, u32 epoch, int rank, int mergers, int tid, MergeScratch<NW>& X) {
   const int wave = tid >> 6, lane = tid & 63;
+  const bool last = blockIdx.x == gridDim.x - 1;
+  // The last block of the grid advances the epoch word for the next launch, once every block of this launch has marked its arrival
+  // (and so has read the word).  The marks' first read is issued here, ahead of the merge work, and looked at after it: by then the
+  // other blocks have long left their loops, so the check normally costs no trip to memory of its own.
+  constexpr int XK = 2048 / (64 * NW);      // marks per lane held in registers: the first 2048 blocks of the grid
+  const u32* marks = A.epochs + EPOCH_WORDS;
+  const int nblocks = (int)gridDim.x, xi = 64 * wave + lane;
+  u32 xm[XK];
+  if (last) {
+#pragma unroll
+    for (int k = 0; k < XK; ++k) xm[k] = __hip_atomic_load(marks + min(xi + 64 * NW * k, nblocks - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
   // The first item stands outside the loop: at a loop header the compiler waits for every memory operation in flight, which here
   // would be the acknowledgement of the block's own record stores (a round trip to memory) before the first record load is issued.
   int item = rank;
   if (item < 2 * G) { merge_half_head<NW>(A, qh0 + (item >> 1), item & 1, epoch, X, wave, lane); item += mergers; }
   for (; item < 2 * G; item += mergers) merge_half_head<NW>(A, qh0 + (item >> 1), item & 1, epoch, X, wave, lane);
-  // the last block of the grid advances the epoch word for the next launch (the blocks of this launch have read it long ago: they
-  // all started before this block did)
-  if (blockIdx.x == gridDim.x - 1 && tid == 0) __hip_atomic_store(A.epochs, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (!last) return;
+  bool grid_ok = true;
+  for (int spin = 0;; ++spin) {
+    bool stale = false;
+#pragma unroll
+    for (int k = 0; k < XK; ++k) stale |= xm[k] != epoch;
+    if (__builtin_amdgcn_ballot_w64(stale) == 0) break;
+    if (spin >= MERGE_SPIN_LIMIT) { grid_ok = false; break; }
+    __builtin_amdgcn_s_sleep(1);
+#pragma unroll
+    for (int k = 0; k < XK; ++k)
+      if (xm[k] != epoch) xm[k] = __hip_atomic_load(marks + min(xi + 64 * NW * k, nblocks - 1), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  for (int i0 = 2048; grid_ok && i0 < nblocks; i0 += 64 * NW) {      // grids beyond 2048 blocks: the remaining marks, a round at a time
+    const int i = min(i0 + xi, nblocks - 1);
+    for (int spin = 0; __builtin_amdgcn_ballot_w64(__hip_atomic_load(marks + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != epoch) != 0; ++spin) {
+      if (spin >= MERGE_SPIN_LIMIT) { grid_ok = false; break; }
+      __builtin_amdgcn_s_sleep(1);
+    }
+  }
+  // The waves' verdicts meet in LDS behind a barrier that orders LDS traffic only: a full block barrier would first wait for the
+  // acknowledgement of the output rows just stored, and the epoch store would then be a second trip to memory at the launch's very end.
+  grid_ok = __builtin_amdgcn_ballot_w64(!grid_ok) == 0;
+  if (lane == 0) X.l[wave][0] = grid_ok ? 1.f : 0.f;
+  lds_barrier();
+  if (tid == 0) {
+    bool all = true;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) all &= X.l[w][0] != 0.f;
+    if (all) __hip_atomic_store(A.epochs, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else merge_failed(A, 2u);
+  }
 }
 
 // ---------------------------------------------------------------------------------------------------- uncompressed rows
@@ -488,9 +545,10 @@ __device__ __forceinline__ void load_tile_escapes(const Bases& B, int lane, cons
   R.k.f = __builtin_amdgcn_ubfe(Tg.kfl, 8 * q, 8); R.v.f = __builtin_amdgcn_ubfe(Tg.vfl, 8 * q, 8);
   R.k.pos0 = (excl & 0xFFFFu) + (u32)esc_prefix(Tg.kfl, 8 * q);
   R.v.pos0 = (excl >> 16) + (u32)esc_prefix(Tg.vfl, 8 * q);
-  if (PAGED) {
-    R.k.e = load_u32x2_unaligned(esc_of_tile<PAGED>(B.kov, __builtin_amdgcn_readfirstlane(Tg.kto), B.TS) + R.k.pos0);
-    R.v.e = load_u32x2_unaligned(esc_of_tile<PAGED>(B.vov, __builtin_amdgcn_readfirstlane(Tg.vto), B.TS) + R.v.pos0);
+  if (PAGED) {      // the 8-byte window stays inside the slot: a lane whose escape bytes start in the slot's last 7 bytes takes the slow look-up
+    const u32 lim = (u32)(B.TS - SLOT_OV - 8);      // TS >= SLOT_OV + 16 (checked on the host)
+    R.k.e = load_u32x2_unaligned(esc_of_tile<PAGED>(B.kov, __builtin_amdgcn_readfirstlane(Tg.kto), B.TS) + min(R.k.pos0, lim));
+    R.v.e = load_u32x2_unaligned(esc_of_tile<PAGED>(B.vov, __builtin_amdgcn_readfirstlane(Tg.vto), B.TS) + min(R.v.pos0, lim));
   } else {      // stream base (uniform) + 32-bit offset (tile offset + position in the tile)
     R.k.pos0 += Tg.kto; R.v.pos0 += Tg.vto;
     R.k.e = load_u32x2_unaligned(B.kov + R.k.pos0);
@@ -536,8 +594,9 @@ __device__ __forceinline__ u32x4 raw_x_words(u32 lo, u32 hi, const u32x4& b4w) {
 // common instantiation has no memory access between the prefetch and the products.
 // bw[u]: the exponent-base words of unit u's tier, read from the block's LDS table: one table row per (tier, group), so the tier
 // select costs an address bit instead of four conditional moves per unit.
+// lim (SLOW only): last offset from esc_tile at which an 8-byte load may start (paged pool: the slot's end - 8; a stream: no limit).
 template <int KIND, bool SLOW>
-__device__ __forceinline__ void unit_x_words(const KindRegs& R, const AttnLds& L, const uint8_t* __restrict__ esc_tile, int a, int q,
+__device__ __forceinline__ void unit_x_words(const KindRegs& R, const AttnLds& L, const uint8_t* __restrict__ esc_tile, u32 lim, int a, int q,
                                              u32x4* __restrict__ x, u32x4* __restrict__ bw) {
   const u32 tag8 = R.f;
   const u32 eb4 = __builtin_amdgcn_perm(R.e[1], R.e[0], L.sel[tag8]);
@@ -547,7 +606,7 @@ __device__ __forceinline__ void unit_x_words(const KindRegs& R, const AttnLds& L
     x[u] = L.xlut[(eb4 >> (8 * u)) & 0xFFu];
     bw[u] = tab[(KIND == KIND_K ? u : 0) + NG * ((tag8 >> (2 * u)) & 1u)];
   }
-  if (__builtin_amdgcn_ballot_w64((tag8 & 0xAAu) != 0u)) {
+  if (__builtin_amdgcn_ballot_w64((tag8 & 0xAAu) != 0u || (SLOW && tag8 != 0u && R.pos0 > lim))) {
     const u64 e64 = (u64)R.e[0] | ((u64)R.e[1] << 32);
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
@@ -556,13 +615,14 @@ __device__ __forceinline__ void unit_x_words(const KindRegs& R, const AttnLds& L
         x[u] = raw_x_words((u32)v, (u32)(v >> 32), bw[u]);
       }
     }
-    if (SLOW && __popc(tag8 & 0xAAu) >= 2) {
+    if (SLOW && (__popc(tag8 & 0xAAu) >= 2 || R.pos0 > lim)) {
       u32 off = 0u;
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
         const u32 t = (tag8 >> (2 * u)) & 3u;
         if (t) {
-          const u64 v = load_u64_unaligned(esc_tile + R.pos0 + off);
+          const u32 at = R.pos0 + off, from = min(at, lim);      // bytes past the limit are not this unit's: load lower, shift down
+          const u64 v = load_u64_unaligned(esc_tile + from) >> (8u * (at - from));
           // The loaded bytes are waited for here, in the block that issues the load: their two users below sit in separate divergent
           // blocks, and a load that is still pending on the path past both makes the compiler wait for every load in flight wherever
           // its register is reused, on the common path as well.
@@ -586,12 +646,15 @@ __device__ __forceinline__ void consume(const TileRegs& R, WaveState& st, const 
   // groups).  The choice is one wave-uniform branch around the look-ups only, ahead of all the matrix products of the tile.
   u32x4 xk[4], xv[4], bk[4], bv[4];
   const u32 kr = R.k.f & 0xAAu, vr = R.v.f & 0xAAu;
-  if (__builtin_expect(__builtin_amdgcn_ballot_w64(((kr & (kr - 1u)) | (vr & (vr - 1u))) != 0u) != 0, 0)) {
-    unit_x_words<KIND_K, true>(R.k, L, PAGED ? esc_of_tile<PAGED>(B.kov, kto, B.TS) : B.kov, a, q, xk, bk);
-    unit_x_words<KIND_V, true>(R.v, L, PAGED ? esc_of_tile<PAGED>(B.vov, vto, B.TS) : B.vov, a, q, xv, bv);
+  const u32 lim = PAGED ? (u32)(B.TS - SLOT_OV - 8) : 0xFFFFFFFFu;      // paged pool: the 8 prefetched bytes were taken from no further than this
+  bool slow = ((kr & (kr - 1u)) | (vr & (vr - 1u))) != 0u;
+  if (PAGED) slow |= (R.k.f != 0u && R.k.pos0 > lim) || (R.v.f != 0u && R.v.pos0 > lim);
+  if (__builtin_expect(__builtin_amdgcn_ballot_w64(slow) != 0, 0)) {
+    unit_x_words<KIND_K, true>(R.k, L, PAGED ? esc_of_tile<PAGED>(B.kov, kto, B.TS) : B.kov, lim, a, q, xk, bk);
+    unit_x_words<KIND_V, true>(R.v, L, PAGED ? esc_of_tile<PAGED>(B.vov, vto, B.TS) : B.vov, lim, a, q, xv, bv);
   } else {
-    unit_x_words<KIND_K, false>(R.k, L, nullptr, a, q, xk, bk);
-    unit_x_words<KIND_V, false>(R.v, L, nullptr, a, q, xv, bv);
+    unit_x_words<KIND_K, false>(R.k, L, nullptr, lim, a, q, xk, bk);
+    unit_x_words<KIND_V, false>(R.v, L, nullptr, lim, a, q, xv, bv);
   }
   // ---- scores: S[tok 4q+r][head a]
   f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
@@ -731,8 +794,9 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
   }
   if (tid < 256) tables_load_bases(Tr, tid, A.k.base3, A.k.base4, A.v.base3, A.v.base4, ch % A.NB);
 
-  const int ntiles = (S + T - 1) / T, chunk = PAGED ? min((ntiles + A.nsplit - 1) / A.nsplit, MAX_CHUNK) : (ntiles + A.nsplit - 1) / A.nsplit;
+  const int ntiles = (S + T - 1) / T, chunk = (ntiles + A.nsplit - 1) / A.nsplit;
   const int tlo = min(split * chunk, ntiles), thi = min(tlo + chunk, ntiles);
+  const int thi_fast = PAGED ? min(thi, tlo + MAX_CHUNK) : thi;      // the pipelined loop's range: what one fill of the LDS tile table covers
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63, a = lane & 15, q = lane >> 4;
   Bases B;
   TileTable TT{tile_table, tlo};
@@ -740,7 +804,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
     // logical tile -> block table -> mode table (paged_kernel.py:137-138), resolved once per block into LDS
     B.kov = B.vov = A.pool; B.TS = A.TS;
     B.ksm = B.kcd = B.vsm = B.vcd = nullptr; B.kfl = B.kto = B.vfl = B.vto = nullptr;
-    for (int i = tid; i < thi - tlo; i += NT) {
+    for (int i = tid; i < thi_fast - tlo; i += NT) {
       const long pc = (long)A.bt[(long)b * A.bt_stride + tlo + i] * (2 * A.n_kv) + 2 * kvh;
       tile_table[i] = int2{A.mt[pc], A.mt[pc + 1]};
     }
@@ -761,8 +825,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
   // branch the consumer has to join) and not consumed.  A partly filled last tile of the sequence is handled at the end by wave 0.
   // logical tile index i of this block -> tile tlo + i
   const int full = ntiles - ((S % T) != 0 ? 1 : 0);      // tiles with all 16 rows
-  const int n_own = max(min(thi, full) - tlo, 0);
-  const bool part_here = (S % T) != 0 && thi == ntiles && thi > tlo;
+  const int n_own = max(min(thi_fast, full) - tlo, 0);
   const int icl = max(n_own - 1, 0);
 #define TILE(i) (tlo + (i))
   int iA = wave, iB = wave + NW;
@@ -838,44 +901,69 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
     }
   }
 #undef TILE
+  // arrival mark of the block for the fused merge (see merge_heads): the wave has no load in flight here
+  if (A.epochs != nullptr && A.nslot > 1 && tid == 0) mark_arrival(A, epoch);
   GAAC_STAMP(2);
 #ifdef GAAC_PHASE_TIMING
   if (A.dbg && lane == 0) A.dbg[((long)gridDim.x + blockIdx.x) * 8 + wave] = wall_clock64();
 #endif
-  if (part_here && wave == 0) {
-    const int t = ntiles - 1;
-    load_tags<PAGED>(B, TT, t, a, Tg);
-    load_tile<PAGED>(B, t, lane, Tg, R0);
-    if (!PAGED || !Tg.raw) consume<PAGED, true>(R0, st, L, B, Tg.kto, Tg.vto, t, S, A.scale_log2e, a, q, qf);
-  }
-  // ---- paged pool: tiles of this split whose K or V side is a raw tile (the block that is still filling, or escapes that did not
-  // fit the slot) are attended by the whole block
-  if (PAGED) {
-    bool mine = false;
-    for (int i = tid; i < thi - tlo; i += NT) mine |= (tile_table[i].x | tile_table[i].y) < 0;
-    if (__syncthreads_or(mine)) {
-      RawScratch& R = *reinterpret_cast<RawScratch*>(&M.acc[0][0][0]);
-      for (int g = tid >> 7; g < G; g += NT / 128) M.acc[NW][g][tid & 127] = 0.f;
-      raw_rows_begin<NT>(R, A, qh0, G, tid);
-      const uint8_t* b3k = A.k.base3 + (long)(ch % A.NB) * D; const uint8_t* b4k = A.k.base4 + (long)(ch % A.NB) * D;
-      const uint8_t* b3v = A.v.base3 + (long)(ch % A.NB) * D; const uint8_t* b4v = A.v.base4 + (long)(ch % A.NB) * D;
-      for (int i = 0; i < thi - tlo; ++i) {
-        const int2 e = tile_table[i];
-        if ((e.x | e.y) >= 0) continue;
-        const u16* krows = R.krows; const u16* vrows = R.vrows;
-        if (e.x < 0) krows = A.raw + (long)(~e.x) * T * D;
-        else if (wave == 0) {
-          const uint8_t* sl = A.pool + (size_t)e.x * (size_t)A.TS;
-          decode_tile_rows<KIND_K>(sl, sl + SLOT_CD, reinterpret_cast<const int*>(sl + SLOT_FL), sl + SLOT_OV, b3k, b4k, lane, T, R.krows, D);
+  // ---- what the pipelined loop left: (1) the partly filled last tile of the sequence; (2) paged pool: a split longer than the LDS tile
+  // table goes on in further rounds of MAX_CHUNK tiles (table refilled); (3) paged pool: tiles whose K or V side is a raw tile (the
+  // block that is still filling, or escapes that did not fit the slot), attended by the whole block round by round, while the table
+  // holds their entries.  Tiles of (1) and (2) are taken by the waves in turn, one at a time without the prefetch pipeline (of the
+  // block's waves some compute while others wait for their tile; both cases are rare), through ONE instantiation of the masking tile
+  // code.
+  if (tlo < thi) {
+    bool raw_started = false;
+    for (int c0 = tlo;;) {
+      const int c1 = PAGED ? min(c0 + MAX_CHUNK, thi) : thi;
+      if (PAGED && c0 != tlo) {
+        __syncthreads();      // everybody is done with the previous round's entries
+        for (int i = tid; i < c1 - c0; i += NT) {
+          const long pc = (long)A.bt[(long)b * A.bt_stride + c0 + i] * (2 * A.n_kv) + 2 * kvh;
+          tile_table[i] = int2{A.mt[pc], A.mt[pc + 1]};
         }
-        if (e.y < 0) vrows = A.raw + (long)(~e.y) * T * D;
-        else if (wave == 1) {
-          const uint8_t* sl = A.pool + (size_t)e.y * (size_t)A.TS;
-          decode_tile_rows<KIND_V>(sl, sl + SLOT_CD, reinterpret_cast<const int*>(sl + SLOT_FL), sl + SLOT_OV, b3v, b4v, lane, T, R.vrows, D);
-        }
-        raw_rows_attend<NT>(R, krows, vrows, min(T, S - (tlo + i) * T), A.scale_log2e, G, tid, M.m[NW], M.l[NW], M.acc[NW]);
-        __syncthreads();      // staging rows are free again
+        __syncthreads();
+        TT.tlo = c0;
       }
+      for (int t = (c0 == tlo ? tlo + n_own : c0) + wave; t < c1; t += NW) {      // first round: only the partial tile is left (wave 0)
+        load_tags<PAGED>(B, TT, t, a, Tg);
+        load_tile<PAGED>(B, t, lane, Tg, R0);
+        if (!PAGED || !Tg.raw) consume<PAGED, true>(R0, st, L, B, Tg.kto, Tg.vto, t, S, A.scale_log2e, a, q, qf);
+      }
+      if (PAGED) {
+        bool mine = false;
+        for (int i = tid; i < c1 - c0; i += NT) mine |= (tile_table[i].x | tile_table[i].y) < 0;
+        if (__syncthreads_or(mine)) {
+          RawScratch& R = *reinterpret_cast<RawScratch*>(&M.acc[0][0][0]);
+          if (!raw_started) {
+            for (int g = tid >> 7; g < G; g += NT / 128) M.acc[NW][g][tid & 127] = 0.f;
+            raw_rows_begin<NT>(R, A, qh0, G, tid);
+            raw_started = true;
+          }
+          const uint8_t* b3k = A.k.base3 + (long)(ch % A.NB) * D; const uint8_t* b4k = A.k.base4 + (long)(ch % A.NB) * D;
+          const uint8_t* b3v = A.v.base3 + (long)(ch % A.NB) * D; const uint8_t* b4v = A.v.base4 + (long)(ch % A.NB) * D;
+          for (int i = 0; i < c1 - c0; ++i) {
+            const int2 e = tile_table[i];
+            if ((e.x | e.y) >= 0) continue;
+            const u16* krows = R.krows; const u16* vrows = R.vrows;
+            if (e.x < 0) krows = A.raw + (long)(~e.x) * T * D;
+            else if (wave == 0) {
+              const uint8_t* sl = A.pool + (size_t)e.x * (size_t)A.TS;
+              decode_tile_rows<KIND_K>(sl, sl + SLOT_CD, reinterpret_cast<const int*>(sl + SLOT_FL), sl + SLOT_OV, b3k, b4k, lane, T, R.krows, D);
+            }
+            if (e.y < 0) vrows = A.raw + (long)(~e.y) * T * D;
+            else if (wave == 1) {
+              const uint8_t* sl = A.pool + (size_t)e.y * (size_t)A.TS;
+              decode_tile_rows<KIND_V>(sl, sl + SLOT_CD, reinterpret_cast<const int*>(sl + SLOT_FL), sl + SLOT_OV, b3v, b4v, lane, T, R.vrows, D);
+            }
+            raw_rows_attend<NT>(R, krows, vrows, min(T, S - (c0 + i) * T), A.scale_log2e, G, tid, M.m[NW], M.l[NW], M.acc[NW]);
+            __syncthreads();      // staging rows are free again
+          }
+        }
+      }
+      c0 = c1;
+      if (c0 >= thi) break;
     }
   }
   // The accumulators are MFMA results: keep their first non-MFMA read a full MFMA latency away on every path.
@@ -894,7 +982,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
       for (int r = 0; r < 4; ++r) M.acc[wave][a][chan_v(8 * (4 * q + r) + i)] = acc[i][r];
   }
   GAAC_MSTAMP(5, wall_clock64());
-  __syncthreads();
+  lds_barrier();      // only LDS data crosses (a full barrier would also wait for the acknowledgement of the arrival mark)
   GAAC_MSTAMP(6, wall_clock64());
   const bool fused = A.epochs != nullptr;
   const int mergers = merge_ranks(G, A.nslot), rank = (int)blockIdx.x % A.nsplit - (A.nsplit - mergers);      // the head's last blocks to start
@@ -1076,6 +1164,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_bf16_attn_split(co
       tA = tC; tB = tD;
     }
   }
+  if (A.nslot > 1 && tid == 0) mark_arrival(A, epoch);
   if (part_here && wave == 0) {
     load_raw_tile(kh, vh, ntiles - 1, S, a, q, R0);
     consume_raw_tile<true>(R0, st, ntiles - 1, S, A.scale_log2e, q, qf);
@@ -1090,7 +1179,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_bf16_attn_split(co
 #pragma unroll
       for (int r = 0; r < 4; ++r) L.acc[wave][a][8 * (4 * q + r) + i] = st.acc[i][r];
   }
-  __syncthreads();
+  lds_barrier();
   const int mergers = merge_ranks(G, A.nslot), rank = split - (A.nsplit - mergers);
   const int d = tid & 127;
   for (int g = tid >> 7; g < G; g += NT / 128) {
@@ -1202,15 +1291,84 @@ extern "C" int gaac_attn_fused(
 }
 
 // ---- the one entry point that allocates nothing ------------------------------------------------------------------------------------
-// gaac_attn_fused with its workspace (partial records + epoch word) in a file-scope device array instead of caller memory, for callers
+// gaac_attn_fused with its workspace (partial records + epoch words) in a file-scope device array instead of caller memory, for callers
 // that cannot allocate: code under HIP graph capture, tight serving loops.  Every GPU the library runs on holds its own copy of the
-// array (4 MiB) from module load to process end; its address on a device comes from hipGetSymbolAddress, once per device.
+// array (4 MiB) from module load to process end; its address on a device comes from hipGetSymbolAddress, once per device
+// (gaac_static_init, or the first call on that device outside stream capture).
 constexpr size_t STATIC_SCRATCH_BYTES = 4u << 20;
-constexpr size_t STATIC_EPOCH_BYTES = 256;                                                  // the epoch word, on a line of its own
-constexpr long STATIC_MAX_RECORD_ROWS = (long)((STATIC_SCRATCH_BYTES - STATIC_EPOCH_BYTES) / ((D + 2) * sizeof(u64)));      // B*n_q*nsplit <= 4032
+constexpr long STATIC_MAX_RECORD_ROWS = 4000;                                               // B*n_q*nsplit (and so the grid's blocks) at most
+constexpr size_t STATIC_EPOCH_BYTES = ((EPOCH_WORDS + STATIC_MAX_RECORD_ROWS) * sizeof(u32) + 255) / 256 * 256;      // epoch words + arrival marks
+static_assert(STATIC_EPOCH_BYTES + STATIC_MAX_RECORD_ROWS * (D + 2) * sizeof(u64) <= STATIC_SCRATCH_BYTES, "the built-in workspace holds 4000 partial rows");
 static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];              // zero at module load: epoch 0, no records
 constexpr int STATIC_MAX_DEVICES = 64;
-static void* g_scratch_ptr[STATIC_MAX_DEVICES];      // the array's address on each device (the name `scratch` is not one in host code)
+static std::atomic<void*> g_scratch_ptr[STATIC_MAX_DEVICES];      // the array's address on each device (the name `scratch` is not one in host code)
+static std::mutex g_scratch_mutex;
+
+// The device a call runs on: the stream's own device when it has one, else the calling thread's current device.
+static int static_device_of(hipStream_t stream, int* dev) {
+  hipDevice_t d = -1;
+  hipError_t e = stream ? hipStreamGetDevice(stream, &d) : hipGetDevice(&d);
+  if (e != hipSuccess || d < 0 || d >= STATIC_MAX_DEVICES) return gaac::fail("gaac static workspace: no usable device (%s)", hipGetErrorString(e));
+  *dev = (int)d;
+  return 0;
+}
+// Resolves (once per device, under a lock) and returns the array's address on `dev`; dev must be the calling thread's current device.
+static int static_scratch(int dev, bool may_resolve, unsigned char** base) {
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (!p) {
+    if (!may_resolve)
+      return gaac::fail("gaac_attn_fused_static: the built-in workspace of device %d has not been set up and the stream is capturing; "
+                        "call gaac_static_init() once before the capture", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    p = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+    if (!p) {
+      int cur = -1;
+      hipError_t e = hipGetDevice(&cur);
+      if (e != hipSuccess || cur != dev) return gaac::fail("gaac static workspace: device %d is not the calling thread's current device (%d)", dev, cur);
+      e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      if (e != hipSuccess || !p) return gaac::fail("gaac static workspace: hipGetSymbolAddress failed (%s)", hipGetErrorString(e));
+      g_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
+  }
+  *base = static_cast<unsigned char*>(p);
+  return 0;
+}
+
+extern "C" int gaac_static_init(void) {
+  int dev = -1;
+  if (int rc = static_device_of(nullptr, &dev)) return rc;
+  unsigned char* base = nullptr;
+  return static_scratch(dev, true, &base);
+}
+
+__global__ void __launch_bounds__(256) k_fill_zero(u32x4* __restrict__ p, long n16) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i < n16) p[i] = u32x4{0u, 0u, 0u, 0u};
+}
+// Re-arms the built-in workspace of the stream's device after a failed launch: epoch words and records back to zero, by a kernel (not
+// a memset node, so the call may be captured).
+extern "C" int gaac_static_reset(void* stream) {
+  int dev = -1;
+  if (int rc = static_device_of((hipStream_t)stream, &dev)) return rc;
+  hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+  if (stream && hipStreamIsCapturing((hipStream_t)stream, &cs) != hipSuccess) cs = hipStreamCaptureStatusNone;
+  unsigned char* base = nullptr;
+  if (int rc = static_scratch(dev, cs == hipStreamCaptureStatusNone, &base)) return rc;
+  const long n16 = (long)(STATIC_SCRATCH_BYTES / 16);
+  hipLaunchKernelGGL(k_fill_zero, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, (hipStream_t)stream, reinterpret_cast<u32x4*>(base), n16);
+  return launch_status("gaac_static_reset");
+}
+// Failure bits of the built-in workspace of the stream's device (see gaac_attn_fused), copied to *flags_out (device memory) on the stream.
+extern "C" int gaac_static_flags(unsigned int* flags_out, void* stream) {
+  GAAC_REQUIRE(flags_out, "gaac_static_flags: null output");
+  int dev = -1;
+  if (int rc = static_device_of((hipStream_t)stream, &dev)) return rc;
+  unsigned char* base = nullptr;
+  if (int rc = static_scratch(dev, true, &base)) return rc;
+  hipError_t e = hipMemcpyAsync(flags_out, base + sizeof(unsigned int), sizeof(unsigned int), hipMemcpyDeviceToDevice, (hipStream_t)stream);
+  if (e != hipSuccess) return gaac::fail("gaac_static_flags: %s", hipGetErrorString(e));
+  return 0;
+}
 
 extern "C" int gaac_attn_fused_static(
     const uint8_t* smk, const uint8_t* ck, const int* fk, const int* tok, const uint8_t* ovk, const int* ohsk, const uint8_t* b3k, const uint8_t* b4k,
@@ -1224,15 +1382,13 @@ extern "C" int gaac_attn_fused_static(
                "gaac_attn_fused_static: B*n_q*nsplit = %ld exceeds the %ld partial rows the built-in workspace (%zu bytes) holds; use gaac_attn_fused with caller memory",
                rec_rows, STATIC_MAX_RECORD_ROWS, STATIC_SCRATCH_BYTES);
   int dev = -1;
-  hipError_t e = hipGetDevice(&dev);
-  if (e != hipSuccess || dev < 0 || dev >= STATIC_MAX_DEVICES) return gaac::fail("gaac_attn_fused_static: no current device (%s)", hipGetErrorString(e));
-  if (!g_scratch_ptr[dev]) {
-    void* p = nullptr;
-    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-    if (e != hipSuccess || !p) return gaac::fail("gaac_attn_fused_static: hipGetSymbolAddress failed (%s)", hipGetErrorString(e));
-    g_scratch_ptr[dev] = p;
+  if (int rc = static_device_of((hipStream_t)stream, &dev)) return rc;
+  unsigned char* base = g_scratch_ptr[dev].load(std::memory_order_acquire) ? static_cast<unsigned char*>(g_scratch_ptr[dev].load(std::memory_order_acquire)) : nullptr;
+  if (!base) {      // first call on this device: resolve the address now, unless the stream is capturing (no runtime query inside a capture)
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (stream && hipStreamIsCapturing((hipStream_t)stream, &cs) != hipSuccess) cs = hipStreamCaptureStatusNone;
+    if (int rc = static_scratch(dev, cs == hipStreamCaptureStatusNone, &base)) return rc;
   }
-  unsigned char* base = static_cast<unsigned char*>(g_scratch_ptr[dev]);
   unsigned int* epoch = reinterpret_cast<unsigned int*>(base);
   unsigned long long* pm = reinterpret_cast<unsigned long long*>(base + STATIC_EPOCH_BYTES);
   unsigned long long* pl = pm + rec_rows;
@@ -1248,11 +1404,10 @@ extern "C" int gaac_paged_attn(
     unsigned long long* pm, unsigned long long* pl, unsigned long long* pa, unsigned int* epoch, void* out, void* stream) {
   GAAC_REQUIRE(n_kv > 0 && n_q > 0 && n_q % n_kv == 0 && n_q / n_kv <= GMAX, "GQA group size must be 1..%d (n_q=%d, n_kv=%d)", GMAX, n_q, n_kv);
   GAAC_REQUIRE(pool && raw && mt && bt && seq_lens && q && b3k && b4k && b3v && b4v && pm && pl && pa && epoch && out, "gaac_paged_attn: null pointer");
-  GAAC_REQUIRE(B > 0 && NB > 0 && TS >= SLOT_OV && TS % 16 == 0 && bt_stride > 0, "gaac_paged_attn: bad sizes B=%d NB=%d TS=%d", B, NB, TS);
+  GAAC_REQUIRE(B > 0 && NB > 0 && TS >= SLOT_OV + 16 && TS % 16 == 0 && bt_stride > 0, "gaac_paged_attn: bad sizes B=%d NB=%d TS=%d (a slot is %d bytes plus at least 16 for escapes)", B, NB, TS, SLOT_OV);
   GAAC_REQUIRE(nsplit >= 1 && nsplit <= MAX_SLOTS, "gaac_paged_attn: nsplit must be in 1..%d", MAX_SLOTS);
   const long max_tiles = ((long)max_seq_len + T - 1) / T;
-  GAAC_REQUIRE(max_seq_len >= 0 && max_tiles <= (long)bt_stride && (max_tiles + nsplit - 1) / nsplit <= MAX_CHUNK,
-               "gaac_paged_attn: max_seq_len %d needs at most %d blocks per row and at least %ld splits", max_seq_len, bt_stride, (max_tiles + MAX_CHUNK - 1) / MAX_CHUNK);
+  GAAC_REQUIRE(max_seq_len >= 0 && max_tiles <= (long)bt_stride, "gaac_paged_attn: max_seq_len %d needs %ld blocks per row, the block table has %d", max_seq_len, max_tiles, bt_stride);
   AttnArgs A;
   A.k = StoreView{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, b3k, b4k};
   A.v = StoreView{nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, b3v, b4v};

@@ -224,12 +224,6 @@ __global__ void __launch_bounds__(64) k_decode_tiles(const uint8_t* __restrict__
                            min(T, S - tile * T), dst, out_row_stride);
 }
 
-// Plain streaming copy with the access shape of the attention kernel's payload loads (16 B per lane, 1 KiB per wave-wide
-// load): the known-size kernel against which HBM traffic counters are calibrated.
-__global__ void __launch_bounds__(256) k_stream_copy(const u32x4* __restrict__ src, u32x4* __restrict__ dst, long n16) {
-  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n16; i += (long)gridDim.x * 256) dst[i] = src[i];
-}
-
 }  // namespace gaac
 
 using namespace gaac;
@@ -295,14 +289,6 @@ int gaac_decode_tiles(int kind, const uint8_t* sm, const uint8_t* codes, const i
   if (kind == 0) hipLaunchKernelGGL(k_decode_tiles<KIND_K>, grid, dim3(64), 0, (hipStream_t)stream, sm, codes, flags, tile_off, ovf, head_start, base3, base4, n_kv, bidx, S, S_pad, (u16*)out, out_head_stride, out_row_stride);
   else hipLaunchKernelGGL(k_decode_tiles<KIND_V>, grid, dim3(64), 0, (hipStream_t)stream, sm, codes, flags, tile_off, ovf, head_start, base3, base4, n_kv, bidx, S, S_pad, (u16*)out, out_head_stride, out_row_stride);
   return launch_status("gaac_decode_tiles");
-}
-
-int gaac_stream_copy(const void* src, void* dst, long nbytes, void* stream) {
-  GAAC_REQUIRE(src && dst && nbytes > 0 && nbytes % 16 == 0, "gaac_stream_copy: nbytes must be a positive multiple of 16");
-  const long n16 = nbytes / 16;
-  const int blocks = (int)((n16 + 255) / 256 < 8192 ? (n16 + 255) / 256 : 8192);
-  hipLaunchKernelGGL(k_stream_copy, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (const u32x4*)src, (u32x4*)dst, n16);
-  return launch_status("gaac_stream_copy");
 }
 
 }  // extern "C"

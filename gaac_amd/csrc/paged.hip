@@ -163,7 +163,7 @@ int gaac_paged_store(const void* key, const void* value, long k_stride, long v_s
                      uint8_t* pool, int TS, void* raw, int* mt, int* stack, int* top, int* err, int* freeq,
                      const uint8_t* b3k, const uint8_t* b4k, const uint8_t* b3v, const uint8_t* b4v, int n_kv, void* stream) {
   GAAC_REQUIRE(key && value && ent && pool && raw && mt && stack && top && err && freeq && b3k && b4k && b3v && b4v, "gaac_paged_store: null pointer");
-  GAAC_REQUIRE(n_ent > 0 && n_kv > 0 && TS >= SLOT_OV && TS % 16 == 0 && k_stride >= (long)n_kv * D && v_stride >= (long)n_kv * D,
+  GAAC_REQUIRE(n_ent > 0 && n_kv > 0 && TS >= SLOT_OV + 16 && TS % 16 == 0 && k_stride >= (long)n_kv * D && v_stride >= (long)n_kv * D,
                "gaac_paged_store: bad sizes n_ent=%d n_kv=%d TS=%d", n_ent, n_kv, TS);
   PagedStoreArgs A{(const u16*)key, (const u16*)value, k_stride, v_stride, ent, n_ent, pool, TS, (u16*)raw, mt, stack, top, err, freeq,
                    b3k, b4k, b3v, b4v, n_kv, TS - SLOT_OV};
@@ -186,7 +186,7 @@ int gaac_paged_release(const int* blocks, int n_blocks, int* mt, int* stack, int
 int gaac_paged_decode(const uint8_t* pool, int TS, const void* raw, const int* mt, const int* pairs, int n_pairs, void* sk, void* sv,
                       long row_stride, const uint8_t* b3k, const uint8_t* b4k, const uint8_t* b3v, const uint8_t* b4v, int n_kv, void* stream) {
   GAAC_REQUIRE(pool && raw && mt && pairs && sk && sv && b3k && b4k && b3v && b4v, "gaac_paged_decode: null pointer");
-  GAAC_REQUIRE(n_pairs > 0 && n_kv > 0 && TS >= SLOT_OV && TS % 16 == 0 && row_stride >= (long)n_kv * D, "gaac_paged_decode: bad sizes");
+  GAAC_REQUIRE(n_pairs > 0 && n_kv > 0 && TS >= SLOT_OV + 16 && TS % 16 == 0 && row_stride >= (long)n_kv * D, "gaac_paged_decode: bad sizes");
   PagedDecodeArgs A{pool, TS, (const u16*)raw, mt, pairs, (u16*)sk, (u16*)sv, row_stride, b3k, b4k, b3v, b4v, n_kv};
   hipLaunchKernelGGL(k_paged_decode, dim3(n_pairs, 2 * n_kv), dim3(64), 0, (hipStream_t)stream, A);
   return launch_status("gaac_paged_decode");

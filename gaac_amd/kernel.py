@@ -61,33 +61,67 @@ def choose_nsplit(B: int, n_kv: int, S: int, target_ctas: int = 256, min_tok: in
 
 
 class AttnWorkspace:
-    """Output + split partials of one launch shape (rows = B*n_q): m, l [rows*NSLOT] and acc [rows*NSLOT*D].  The one-kernel launch
-    stores every partial value as a 64-bit record (fp32 bits | launch epoch << 32); the two-kernel launch writes plain fp32 into the
-    front of the same buffers.  epoch: one word, the epoch of the last merged one-kernel launch on this workspace."""
+    """Output + split partials of one launch shape (rows = B*n_q).  The one-kernel launch stores every partial value as a 64-bit
+    record (fp32 bits | launch epoch << 32): pm, pl [rows*NSLOT], pa [rows*NSLOT*D] int64.  epoch: [0] the epoch of the last merged
+    one-kernel launch on this workspace, [1] failure bits that a launch sets instead of hanging (bit 0: a merging block gave up
+    waiting for a partial and wrote its rows as NaN; bit 1: the epoch could not be advanced), [2 + i] the arrival mark of block i of
+    the launch (rows*NSLOT words: a launch has B*n_kv*NSLOT <= rows*NSLOT blocks).  The two-kernel launch
+    (phase "split" / "combine" / "both") keeps plain fp32 partials in buffers of its own, made on first use, so that its values can
+    never be taken for records."""
     def __init__(self, rows: int, nslot: int, dtype, dev, with_out: bool = True):
-        self.rows, self.nslot = rows, nslot
+        self.rows, self.nslot, self.dev = rows, nslot, dev
         self.out = torch.empty(rows, D, dtype=dtype, device=dev) if with_out else None      # None: a fresh output per launch
         self.pm = torch.zeros(rows * nslot, dtype=torch.int64, device=dev)
         self.pl = torch.zeros(rows * nslot, dtype=torch.int64, device=dev)
         self.pa = torch.zeros(rows * nslot * D, dtype=torch.int64, device=dev)
-        self.epoch = torch.zeros(1, dtype=torch.int32, device=dev)
+        self.epoch = torch.zeros(2 + rows * nslot, dtype=torch.int32, device=dev)
+        self._f32 = None
+
+    def f32_partials(self):
+        """fp32 pm, pl, pa of the two-kernel launch (allocated on first use)."""
+        if self._f32 is None:
+            n = self.rows * self.nslot
+            self._f32 = tuple(torch.empty(k, dtype=torch.float32, device=self.dev) for k in (n, n, n * D))
+        return self._f32
+
+    def failure_bits(self) -> int:
+        """Host read of the failure word (synchronizes with the device)."""
+        return int(self.epoch[1])
+
+    def check(self):
+        """Raises if a one-kernel launch on this workspace gave up a wait since the last reset() (its output rows are NaN, or the
+        epoch stands still); poll it where the engine polls its other device-side error words."""
+        bits = self.failure_bits()
+        if bits:
+            raise RuntimeError("fused decode attention gave up waiting for" + (" a split's partial (rows written as NaN)" if bits & 1 else "") +
+                               (" the other blocks of the launch (epoch not advanced)" if bits & 2 else "") +
+                               "; the workspace may hold records of a wrong epoch: re-arm with reset()")
 
     def reset(self):
-        """Re-arm after a failed launch: the epochs and the records start from zero again."""
+        """Re-arm after a failed launch: the epochs, the failure bits and the records start from zero again."""
         for t in (self.pm, self.pl, self.pa, self.epoch): t.zero_()
 
 
+_SHARED_WS_MAX = 8            # launch shapes whose workspace is kept per process; the least recently used one goes first
 _shared_ws: dict = {}
 
 
 def shared_workspace(rows: int, nslot: int, dtype, dev) -> AttnWorkspace:
     """The workspace that callers who pass none share: one per (device, launch shape, stream), zeroed once when it is made (a fresh
-    buffer per call would have to be cleared per call: recycled memory may hold records whose epoch matches a new counter).
-    It has no output buffer of its own, so every launch returns a fresh tensor."""
+    buffer per call would have to be cleared per call: recycled memory may hold records whose epoch matches a new counter), at most
+    _SHARED_WS_MAX of them (least recently used first out).  It has no output buffer of its own, so every launch returns a fresh
+    tensor.  A workspace is never made while the stream is capturing (its memory and its zeroing would end up inside the graph):
+    callers that capture pass their own, as CompressedKVCache and LayerState do."""
     dev = torch.device(dev)
     key = (dev.type, dev.index if dev.index is not None else torch.cuda.current_device(), rows, nslot, dtype, torch.cuda.current_stream(dev).cuda_stream)
-    ws = _shared_ws.get(key)
-    if ws is None: ws = _shared_ws[key] = AttnWorkspace(rows, nslot, dtype, dev, with_out=False)
+    ws = _shared_ws.pop(key, None)
+    if ws is None:
+        if torch.cuda.is_current_stream_capturing():
+            raise RuntimeError("no attention workspace for this launch shape yet and the stream is capturing: run the launch once before "
+                               "the capture, or pass a workspace (AttnWorkspace) of your own")
+        ws = AttnWorkspace(rows, nslot, dtype, dev, with_out=False)
+        while len(_shared_ws) >= _SHARED_WS_MAX: _shared_ws.pop(next(iter(_shared_ws)))
+    _shared_ws[key] = ws      # most recently used last
     return ws
 
 
@@ -117,14 +151,15 @@ def attn_launch(K, V, q2d, slots, n_q, n_kv, SL, S_pad, scale, nsplit, kt=None, 
     p = _lib.ptr
     out = ws.out if ws.out is not None else torch.empty(B * n_q, D, dtype=q2d.dtype, device=q2d.device)
     if phase == "combine":
-        _lib.call("gaac_attn_combine", p(ws.pm), p(ws.pl), p(ws.pa), p(out), B * n_q, nslot, _lib.stream())
+        pm, pl, pa = ws.f32_partials()
+        _lib.call("gaac_attn_combine", p(pm), p(pl), p(pa), p(out), B * n_q, nslot, _lib.stream())
         return out
     args = (*_store_args(K), *_store_args(V), p(q2d), p(slots), B, n_q, n_kv, p(SL), S_pad, float(scale), nsplit, K.base3.shape[0],
             p(kt) if has_tail else None, p(vt) if has_tail else None, p(TL) if has_tail else None, TCAP if has_tail else 0)
     if phase == "fused":
         _lib.call("gaac_attn_fused", *args, int(S_all), p(ws.pm), p(ws.pl), p(ws.pa), p(ws.epoch), p(out), _lib.stream())
         return out
-    args = (*args, p(ws.pm), p(ws.pl), p(ws.pa))
+    args = (*args, *(p(t) for t in ws.f32_partials()))
     if phase == "split":
         _lib.call("gaac_attn_split", *args, _lib.stream())
     else:

@@ -160,7 +160,8 @@ class CompressedKVCache:
         """Host-side guard of the escape windows (kv_cache.py:198-203); the engine calls it every 16 decode steps at the latest.  In
         16 steps a head completes one tile at most, and a tile has at most TILE_MAX_ESC escape bytes, so a window that has that
         much room left after a check cannot fill up before the next one.  Grows the windows when the room is gone; raises if the
-        append kernel already had to drop data.  used: max_escape_bytes() if the caller fetched it already."""
+        append kernel already had to drop data or a fused attention launch gave up waiting for a partial.  used: max_escape_bytes() if the caller fetched it already."""
+        for ws in self._partials.values(): ws.check()      # a fused attention launch that gave up a wait (rows NaN): re-arm with ws.reset()
         hit = int(self.overflow)
         if hit:
             raise RuntimeError("compressed KV cache lost data:" + (" a sequence grew past the slot's token capacity;" if hit & 1 else "") +

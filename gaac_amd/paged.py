@@ -14,15 +14,14 @@ from .kernel import AttnWorkspace, shared_workspace
 D = 128
 BLOCK = 16
 SM_OFF, CD_OFF, FL_OFF, OVF_OFF = 0, 2048, 2816, 2880   # byte layout of a tile slot; TS = OVF_OFF + ovf_slot
-MAX_TILES_PER_SPLIT = 1024
 
 
 def choose_nsplit(B: int, n_kv: int, S: int, target_ctas: int = 2048, min_tok: int = 256, cap: int = 256) -> int:
     """Splits per (row, kv head) for the longest sequence S of the batch: sequences of a serving batch differ in length, so the
     launch is cut into several times more blocks than the 512 that are resident (they balance out as they are scheduled), at
-    least min_tok tokens each, and never more than 1024 tiles per split (the kernel keeps one split's slot lookups in LDS)."""
-    need = -(-(-(-S // BLOCK)) // MAX_TILES_PER_SPLIT)
-    return max(min(max(1, target_ctas // (B * n_kv)), max(1, S // min_tok), cap), need, 1)
+    least min_tok tokens each.  (Any split count works; a split of more than 1024 tiles leaves the prefetch pipeline after its
+    first 1024 and is slower from there on.)"""
+    return max(min(max(1, target_ctas // (B * n_kv)), max(1, S // min_tok), cap), 1)
 
 
 def build_store_entries(num_computed, query_len, block_table) -> np.ndarray:
@@ -44,12 +43,12 @@ def build_store_entries(num_computed, query_len, block_table) -> np.ndarray:
 
 class LayerState:
     """Per-layer device state outside the block pool: raw side pool, mode table, free stack, error counter and bases.  The block pool
-    itself is the caller's allocation; it must be pool_bytes() long, i.e. reach 16 bytes past its last tile slot (at least 8 are
-    required: the kernels fetch escape bytes with unaligned 8-byte loads that may start at the last byte of a slot)."""
+    itself is the caller's allocation of num_blocks * 2 * n_kv slots of TS bytes (pool_bytes()); no kernel touches a byte outside
+    the slots, so an engine's own block buffer of exactly that size can be handed over."""
     def __init__(self, num_blocks: int, n_kv: int, raw_tiles: int, bases: dict, ovf_slot: int = 128, device="cuda"):
         _lib.load()
         self.n_kv, self.ovf_slot, self.TS = n_kv, ovf_slot, OVF_OFF + ovf_slot
-        assert self.TS % 16 == 0, "ovf_slot must be a multiple of 16"
+        assert ovf_slot >= 16 and self.TS % 16 == 0, "ovf_slot must be a positive multiple of 16"
         self.num_blocks = num_blocks
         i32 = dict(dtype=torch.int32, device=device)
         self.mt = torch.arange(num_blocks * 2 * n_kv, **i32)                 # every tile starts 'compressed at itself'
@@ -62,9 +61,8 @@ class LayerState:
 
     @staticmethod
     def pool_bytes(num_blocks: int, n_kv: int, ovf_slot: int = 128) -> int:
-        """Bytes of the block pool: the slots plus 16 bytes of slack (the attention kernel fetches a lane's escape bytes as one
-        unaligned 8-byte load, which may reach up to 7 bytes past the last slot)."""
-        return num_blocks * 2 * n_kv * (OVF_OFF + ovf_slot) + 16
+        """Bytes of the block pool: num_blocks * 2 * n_kv slots of 2880 + ovf_slot bytes, nothing more."""
+        return num_blocks * 2 * n_kv * (OVF_OFF + ovf_slot)
 
     @property
     def bases(self):
@@ -106,6 +104,7 @@ class LayerState:
 
     def check(self):
         """Host poll (every 16 steps in the reference, backend.py:233-236): raises when the raw side pool ran dry."""
+        for ws in self._ws.values(): ws.check()      # a fused attention launch that gave up a wait: re-arm with ws.reset()
         failed = int(self.err)
         if failed:
             raise RuntimeError(f"raw side pool exhausted ({failed} failed allocations); raise raw_tiles or ovf_slot")
@@ -122,8 +121,7 @@ class LayerState:
 def paged_attention(q, out, buf, raw, mt, bt, seq_lens, bases, TS, n_q, n_kv, nsplit, max_seq_len=None, ws=None):
     """q: [B, n_q, 128] bf16 contiguous; out: [B, n_q*128] bf16 (written); buf: uint8 flat block pool; raw: [tiles,16,128] bf16;
     mt: int32 [num_blocks*2*n_kv]; bt: int32 [B, max_blocks]; seq_lens: int32 [B]; bases: (b3k,b4k,b3v,b4v) uint8 [n_kv,128].
-    max_seq_len: host-side bound of seq_lens (default: what the block table can address).  buf must extend at least 8 bytes past its
-    last tile slot (LayerState.pool_bytes includes 16): escape bytes are fetched with unaligned 8-byte loads.  ws: the launch's
+    max_seq_len: host-side bound of seq_lens (default: what the block table can address).  ws: the launch's
     AttnWorkspace (default: one cached per device, stream and launch shape, so repeated calls allocate nothing)."""
     B = q.shape[0]
     if q.shape[-1] != D: raise RuntimeError("head_dim must be 128")

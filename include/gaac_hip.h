@@ -80,13 +80,18 @@ int gaac_attn_combine(const float* pm, const float* pl, const float* pa, void* o
 
 /* gaac_attn_launch as ONE kernel: the merge of the NSLOT partials (gaac_combine, kernel.py:281-294) is done inside the split kernel
  * by the last (up to sixteen) blocks of each (batch row, kv head) in index order, each taking a share of the head's output, without
- * atomics.  *epoch holds the epoch of the last merged launch; this launch's epoch is that + 1.  Partials travel as 64-bit records
+ * atomics.  epoch[0] holds the epoch of the last merged launch; this launch's epoch is that + 1.  Partials travel as 64-bit records
  * (fp32 bits | epoch << 32) written and read with single 64-bit accesses, so a merging block recognises the records of this launch
- * without waiting for an acknowledgement; it re-reads records that have not arrived yet (bounded; rows are written as NaN if they
- * never do).  The last block of the grid stores the new epoch as its last action.
- * pm, pl: records [B*n_q*nsplit]; pa: records [B*n_q*nsplit*128]; epoch: one uint32.  Zero epoch, pm, pl and pa before the first
+ * without waiting for an acknowledgement; it re-reads records that have not arrived yet.  Every block stores the epoch it works
+ * under into its arrival mark epoch[2 + block] when its first wave is through its tiles; the last block of the grid stores the new
+ * epoch as its last action, after it has seen the marks of all blocks (so every block has read the word).  Every wait is bounded (about 0.1 s): instead of hanging, a launch ORs failure bits into epoch[1]: 1 = a merging block gave
+ * up waiting for a partial and wrote its rows as NaN, 2 = the last block gave up waiting for the other blocks and left epoch[0]
+ * alone.  Poll epoch[1] where the caller polls its other device-side error words.
+ * pm, pl: records [B*n_q*nsplit]; pa: records [B*n_q*nsplit*128]; epoch: uint32 [2 + B*n_kv*nsplit] (epoch word, failure bits, one
+ * arrival mark per block of the launch).  Zero epoch, pm, pl and pa before the first
  * launch and to re-arm them after a failed launch.  Launches of any shape may share them (buffers sized for the largest) as long as
- * they are ordered on one stream.
+ * they are ordered on one stream.  The fp32 partial buffers of gaac_attn_split / gaac_attn_launch must be other memory than these
+ * records (plain values could be taken for records of some epoch).
  * S_all >= 0: every cache head the launch addresses holds exactly S_all compressed tokens (a Page: lengths are known to the host);
  * SL is then not read and may be NULL, which takes one dependent load off the start of every block.  S_all < 0: lengths come from SL. */
 int gaac_attn_fused(
@@ -97,11 +102,20 @@ int gaac_attn_fused(
     unsigned long long* pm, unsigned long long* pl, unsigned long long* pa, unsigned int* epoch, void* out, void* stream);
 
 /* gaac_attn_fused for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that forbid it): the
- * same launch, but the partial records and the epoch word live in a 4 MiB array built into the library (one copy per GPU, held from
+ * same launch, but the partial records and the epoch words live in a 4 MiB array built into the library (one copy per GPU, held from
  * load to process end) instead of caller memory; the call itself allocates nothing.  It has no counterpart in the reference, whose
- * entry allocates its partials on every call (kernel.py:306-307).  Limit: B*n_q*nsplit <= 4032 partial rows (the headline launch uses
+ * entry allocates its partials on every call (kernel.py:306-307).  Limit: B*n_q*nsplit <= 4000 partial rows (the headline launch uses
  * 1024); larger launches are rejected with -1 and a message.  All calls on one GPU share the array: they must be ordered on one
- * stream (calls that overlap on a GPU race), and nothing needs clearing between them (the epoch tells launches apart). */
+ * stream (calls that overlap on a GPU race), and nothing needs clearing between them (the epoch tells launches apart).  The array
+ * of the stream's device is used (the calling thread's current device for the null stream); that device must be the calling
+ * thread's current one when its array is first touched.  The first touch is a runtime query that cannot run while a stream is
+ * capturing: call gaac_static_init() (no arguments, current device, any time before the capture), or make one call outside the
+ * capture; a first call from inside a capture is rejected with a message.
+ * gaac_static_flags copies the array's failure bits (epoch[1] of gaac_attn_fused) to *flags_out (device memory) on the stream;
+ * gaac_static_reset re-arms the array after a failed launch (epoch words and records to zero, by a kernel, so it can be captured). */
+int gaac_static_init(void);
+int gaac_static_reset(void* stream);
+int gaac_static_flags(unsigned int* flags_out, void* stream);
 int gaac_attn_fused_static(
     const uint8_t* smk, const uint8_t* ck, const int* fk, const int* tok, const uint8_t* ovk, const int* ohsk, const uint8_t* b3k, const uint8_t* b4k,
     const uint8_t* smv, const uint8_t* cv, const int* fv, const int* tov, const uint8_t* ovv, const int* ohsv, const uint8_t* b3v, const uint8_t* b4v,
@@ -124,8 +138,8 @@ int gaac_cache_append(
 /* ---- paged slot pool (the layout of /root/reference/gaac/vllm/paged_kernel.py:3-6 and store.py:17-19) -------------------------------
  * pool: tile slots of TS bytes, physical tile p = block*2*n_kv + 2*kvh + kind: [0,2048) sign/mantissa | [2048,2816) codes |
  * [2816,2880) 16 tag words | [2880,TS) escape bytes.  mt int32 [num_blocks*2*n_kv]: p = compressed in its slot, ~r = raw BF16 tile r of
- * raw [tiles][16][128].  stack/top: free raw tiles; err: failed pops.  Bases uint8 [n_kv,128].  The pool allocation must extend at
- * least 8 bytes past its last slot (escape bytes are fetched with unaligned 8-byte loads). */
+ * raw [tiles][16][128].  stack/top: free raw tiles; err: failed pops.  Bases uint8 [n_kv,128].  TS >= 2896 (a slot with no room for
+ * escape bytes would hold no tile the raw pool could not).  No kernel reads or writes outside the slots. */
 
 /* LayerState.store -> _store_tiles, store.py:22-105.  key/value: bf16 rows [num_tokens][n_kv][128] with row strides in elements;
  * ent int32 [n_ent][4] = (block, first token row, offset in block, rows), block < 0 = inactive; freeq int32 [n_ent*2*n_kv] receives
@@ -143,8 +157,9 @@ int gaac_paged_decode(const uint8_t* pool, int TS, const void* raw, const int* m
                       long row_stride, const uint8_t* b3k, const uint8_t* b4k, const uint8_t* b3v, const uint8_t* b4v, int n_kv, void* stream);
 /* paged_attention -> gaac_vpaged_launch, paged_kernel.py:42-277: decode attention of B rows over the pool through the block table
  * bt int32 [B][bt_stride] and the mode table; seq_lens int32 [B] (tokens incl. the filling block; no separate tail); max_seq_len =
- * an upper bound of seq_lens known to the host (bounds the tiles per split, at most 1024).  Partial records pm, pl [B*n_q*nsplit],
- * pa [B*n_q*nsplit*128] and the epoch word as in gaac_attn_fused; out bf16 [B*n_q][128]. */
+ * an upper bound of seq_lens known to the host (checked against the block table's width).  Any nsplit >= 1 works for any length (a
+ * block resolves 1024 tiles of its split at a time).  Partial records pm, pl [B*n_q*nsplit], pa [B*n_q*nsplit*128] and the epoch
+ * buffer [2 + B*n_kv*nsplit] as in gaac_attn_fused; out bf16 [B*n_q][128]. */
 int gaac_paged_attn(const uint8_t* pool, int TS, const void* raw, const int* mt, const int* bt, int bt_stride, const int* seq_lens,
                     int max_seq_len, const void* q, int B, int n_q, int n_kv, float scale, int nsplit,
                     const uint8_t* b3k, const uint8_t* b4k, const uint8_t* b3v, const uint8_t* b4v, int NB,
@@ -158,20 +173,6 @@ int gaac_paged_attn(const uint8_t* pool, int TS, const void* raw, const int* mt,
 int gaac_bf16_attn(const void* k, const void* v, int S, const int* seq_lens, long head_stride_tokens, const void* q, int B, int n_q,
                    int n_kv, float scale, int nsplit, unsigned long long* pm, unsigned long long* pl, unsigned long long* pa,
                    unsigned int* epoch, void* out, void* stream);
-
-/* Measurement aid with no counterpart in the reference: a plain copy of nbytes (multiple of 16) with 16-byte accesses per lane,
- * the known-size kernel that HBM traffic counters (FETCH_SIZE / WRITE_SIZE) are scaled against. */
-int gaac_stream_copy(const void* src, void* dst, long nbytes, void* stream);
-
-/* Measurement aid with no counterpart in the reference: the memory side of gaac_attn_fused without its arithmetic.  One eight-wave
- * block per (cache head, split) streams the K and V page tensors (the first twelve arguments of gaac_attn_fused, without the bases) of
- * H heads x S tokens (S a multiple of 16) with the attention kernel's own loads, one tile ahead; with_meta != 0 adds the tag words,
- * tile offsets and the per-lane escape bytes.  Its duration is the floor the load pattern itself sets under the attention kernel on
- * the same page.  sink: one uint32 (practically never written). */
-int gaac_read_probe(
-    const uint8_t* smk, const uint8_t* ck, const int* fk, const int* tok, const uint8_t* ovk, const int* ohsk,
-    const uint8_t* smv, const uint8_t* cv, const int* fv, const int* tov, const uint8_t* ovv, const int* ohsv,
-    int H, int S, int S_pad, int nsplit, int with_meta, unsigned int* sink, void* stream);
 
 #ifdef __cplusplus
 }

@@ -67,8 +67,8 @@ def test_result_does_not_depend_on_the_split_count():
 def test_fused_merge_equals_the_two_kernel_launch_on_a_reused_workspace():
     """One-kernel launch (one block of each kv head merges) vs split kernel + merge kernel: same partials, so the outputs agree to the
     last bf16 bit or one ulp of rounding order.  Launched several times on one workspace, alternating with the two-kernel launch that
-    overwrites the same buffers with plain fp32: the workspace's epoch word counts the merged launches and the epoch in every
-    record keeps launches apart.  reset() re-arms the workspace."""
+    keeps plain fp32 partials in buffers of its own: the workspace's epoch word counts the merged launches and the epoch in every
+    record keeps launches apart; no launch sets a failure bit.  reset() re-arms the workspace."""
     dev = require_gpu()
     from gaac_amd.kernel import attn_launch, AttnWorkspace
     for (B, n_kv, G, S, ns) in [(1, 8, 4, 4096, 16), (2, 2, 16, 1000, 7), (3, 2, 1, 16, 1), (1, 8, 4, 8192, 64), (1, 2, 4, 3000, 100)]:
@@ -85,11 +85,12 @@ def test_fused_merge_equals_the_two_kernel_launch_on_a_reused_workspace():
             for _ in range(3):
                 one = run("fused", S_all=S if rnd == 1 else -1); n += 1
                 assert (one - two).abs().max().item() <= 2.0 ** -7 * two.abs().max().item()
-            assert int(ws.epoch) == (n if ns > 1 else 0)
+            assert int(ws.epoch[0]) == (n if ns > 1 else 0) and ws.failure_bits() == 0
             assert (run("both") - two).abs().max().item() == 0.0
         ws.reset()
         assert (run("fused") - two).abs().max().item() <= 2.0 ** -7 * two.abs().max().item()
-        assert int(ws.epoch) == (1 if ns > 1 else 0)
+        assert int(ws.epoch[0]) == (1 if ns > 1 else 0)
+        ws.check()
 
 
 def test_epoch_counter_wraps_past_zero():
@@ -105,10 +106,10 @@ def test_epoch_counter_wraps_past_zero():
     run = lambda ph: attn_launch(kp, vp, q, None, n_q, n_kv, SL, kp.sm.shape[1] // 128, SCALE, ns, ws=ws, phase=ph, S_all=S).float().clone()
     two = run("both")
     ws.reset()
-    ws.epoch.fill_(-3)      # 0xFFFFFFFD
+    ws.epoch[0] = -3      # 0xFFFFFFFD
     for want in (-2, -1, 1, 2):
         assert (run("fused") - two).abs().max().item() <= 2.0 ** -7 * two.abs().max().item()
-        assert int(ws.epoch) == want
+        assert int(ws.epoch[0]) == want and ws.failure_bits() == 0
 
 
 def test_launch_shapes_that_share_a_workspace_do_not_mix_their_records():
@@ -290,3 +291,115 @@ def test_bad_arguments_raise():
         attention(torch.zeros(1, 2 * 17, 128, dtype=torch.bfloat16, device=dev), kp, vp, SCALE)
     with pytest.raises(RuntimeError, match="head_dim"):
         attention(torch.zeros(1, 4, 64, dtype=torch.bfloat16, device=dev), kp, vp, SCALE)
+
+
+def test_failure_word_of_a_workspace_raises_and_reset_rearms():
+    """A launch that gives up a wait ORs a bit into the workspace's failure word instead of hanging; the host sees it through
+    AttnWorkspace.check(), CompressedKVCache.check_capacity() and LayerState.check().  The word is set from the host here (no kernel
+    is made to wait on purpose); reset() clears it, and a launch after reset() is right again."""
+    dev = require_gpu()
+    from gaac_amd import CompressedKVCache
+    from gaac_amd.kernel import attn_launch, AttnWorkspace
+    from gaac_amd.paged import LayerState
+    B, n_kv, G, S, ns = 1, 2, 4, 512, 4
+    _, _, kp, vp = _pages(B, n_kv, S, dev, seed=77)
+    n_q = n_kv * G
+    q = to_bf16(randn_bf16((B * n_q, 128), seed=9, scale=0.3), dev)
+    SL = torch.full((B * n_kv,), S, dtype=torch.int32, device=dev)
+    ws = AttnWorkspace(B * n_q, ns, torch.bfloat16, dev)
+    run = lambda: attn_launch(kp, vp, q, None, n_q, n_kv, SL, kp.sm.shape[1] // 128, SCALE, ns, ws=ws, S_all=S).float().clone()
+    want = run()
+    ws.check()
+    assert ws.failure_bits() == 0 and int(ws.epoch[0]) == 1
+    for bits, what in ((1, "partial"), (2, "epoch not advanced"), (3, "partial")):
+        ws.epoch[1] = bits
+        with pytest.raises(RuntimeError, match=what) as ei:
+            ws.check()
+        assert "reset()" in str(ei.value)
+        ws.reset()
+        ws.check()
+        assert int(ws.epoch[0]) == 0 and int(ws.pm.abs().max()) == 0
+        assert torch.equal(run(), want)
+    # the owners of workspaces poll it with their own error words
+    cache = CompressedKVCache(1, n_kv, 64, device=dev)
+    k = to_bf16(randn_bf16((20, n_kv, 128), seed=1), dev)
+    cache.prefill(0, k, k)
+    slots = torch.zeros(1, dtype=torch.int32, device=dev)
+    cache.attention(q.view(1, n_q, 128), slots, SCALE)
+    cache.check_capacity()
+    next(iter(cache._partials.values())).epoch[1] = 1
+    with pytest.raises(RuntimeError, match="reset"):
+        cache.check_capacity()
+    from test_gpu_paged import _bases
+    st = LayerState(4, 4, 8, _bases(dev), 128, dev)
+    st._ws[(1, 16, 1)] = AttnWorkspace(16, 1, torch.bfloat16, dev, with_out=False)
+    st.check()
+    st._ws[(1, 16, 1)].epoch[1] = 2
+    with pytest.raises(RuntimeError, match="reset"):
+        st.check()
+
+
+def test_a_grid_several_times_larger_than_the_gpu_advances_the_epoch_once_per_launch():
+    """Blocks of a grid that does not fit the GPU start as CUs free up, XCD by XCD; the epoch word may only move once every block of the
+    launch has read it.  2 kv heads x 3 splits x 400 rows = 2400 blocks of unequal length (rows with 16 tokens next to rows with 2000,
+    so the last blocks of the grid finish long before others have started), launched repeatedly on one workspace: every launch must
+    agree with the two-kernel launch, advance the epoch by exactly one and set no failure bit."""
+    dev = require_gpu()
+    from gaac_amd import CompressedKVCache
+    n_kv, G, B = 2, 4, 400
+    n_q = n_kv * G
+    cache = CompressedKVCache(B, n_kv, 2048, device=dev)
+    gen = torch.Generator(device=dev).manual_seed(5)
+    lens = [2000 if b % 7 == 0 else 16 + (b % 5) for b in range(B)]
+    for b, L in enumerate(lens):
+        k = (torch.randn(L, n_kv, 128, generator=gen, device=dev)).to(torch.bfloat16); v = (torch.randn(L, n_kv, 128, generator=gen, device=dev)).to(torch.bfloat16)
+        cache.prefill(b, k, v)
+    slots = torch.arange(B, dtype=torch.int32, device=dev)
+    q = (torch.randn(B, n_q, 128, generator=gen, device=dev) * 0.3).to(torch.bfloat16)
+    from gaac_amd.kernel import attn_launch
+    from gaac_amd.kv_cache import TAIL
+    ref = None
+    for rnd in range(6):
+        out = cache.attention(q, slots, SCALE, nsplit=3).float()
+        ws = cache._partials[(B, n_q, 3)]
+        if ref is None:
+            ref = attn_launch(cache.k, cache.v, q.reshape(B * n_q, 128), slots, n_q, n_kv, cache.S, cache.cap, SCALE, 3, cache.k.tail, cache.v.tail,
+                              cache.tail_len, TAIL, ws=ws, phase="both").float().view(B, n_q, 128).clone()
+        assert torch.isfinite(out).all()
+        assert (out - ref).abs().max().item() <= 2.0 ** -7 * ref.abs().max().item()
+        assert int(ws.epoch[0]) == rnd + 1 and ws.failure_bits() == 0
+    cache.check_capacity()
+
+
+def test_headline_size_meets_the_absolute_bar_on_a_spread_softmax():
+    """Config 1's shape (32 query / 8 kv heads, 65536 compressed tokens + 7 raw tail tokens) on unit-scale K and V with a query small
+    enough that the softmax spreads over thousands of rows: the absolute bar max-abs <= 1e-2 and mean-abs <= 1e-3 against fp32 softmax
+    attention (torch, on the device) over the rows that went in.  (The benchmark's own inputs, with channel scales up to 2^4 and
+    outliers x 2^12, make the softmax one-hot.)"""
+    dev = require_gpu()
+    from gaac_amd import Codec, TileEncoder
+    from gaac_amd.kernel import attn_launch, AttnWorkspace, choose_nsplit
+    n_kv, G, S, tail = 8, 4, 65536, 7
+    n_q = n_kv * G
+    gen = torch.Generator(device=dev).manual_seed(21)
+    k = torch.randn(n_kv, S + tail, 128, generator=gen, device=dev); v = torch.randn(n_kv, S + tail, 128, generator=gen, device=dev)
+    # a few far-off small values per row so that all three tiers occur, without weight in the sums
+    hit = torch.rand(n_kv, S + tail, 128, generator=gen, device=dev) < 0.002
+    k = torch.where(hit, k * 2.0 ** -14, k).to(torch.bfloat16); v = torch.where(hit, v * 2.0 ** -14, v).to(torch.bfloat16)
+    ck, cv = Codec(n_kv).calibrate(k[:, :1024]), Codec(n_kv).calibrate(v[:, :1024])
+    kp = TileEncoder("k").encode(ck, k[:, :S].contiguous()); vp = TileEncoder("v").encode(cv, v[:, :S].contiguous())
+    assert torch.equal(Codec.decode(kp).view(torch.int16), k[:, :S].view(torch.int16)) and torch.equal(Codec.decode(vp).view(torch.int16), v[:, :S].view(torch.int16))
+    kt = torch.zeros(n_kv, 16, 128, dtype=torch.bfloat16, device=dev); vt = torch.zeros_like(kt)
+    kt[:, :tail] = k[:, S:]; vt[:, :tail] = v[:, S:]
+    TL = torch.full((n_kv,), tail, dtype=torch.int32, device=dev); SL = torch.full((n_kv,), S, dtype=torch.int32, device=dev)
+    q = (torch.randn(n_q, 128, generator=gen, device=dev) * 0.5).to(torch.bfloat16)
+    sc = torch.einsum("hgd,hsd->hgs", q.float().view(n_kv, G, 128), k.float()) * SCALE
+    p = torch.softmax(sc, -1)
+    assert p.amax(-1).mean().item() < 0.05      # spread: no row carries more than a few percent of a head's weight on average
+    ref = torch.einsum("hgs,hsd->hgd", p, v.float()).reshape(n_q, 128)
+    for ns in (choose_nsplit(1, n_kv, S), 8):
+        ws = AttnWorkspace(n_q, ns, torch.bfloat16, dev)
+        out = attn_launch(kp, vp, q, None, n_q, n_kv, SL, kp.sm.shape[1] // 128, SCALE, ns, kt, vt, TL, 16, ws=ws, S_all=S).float()
+        err = (out - ref).abs()
+        assert err.max().item() <= 1e-2 and err.mean().item() <= 1e-3, (ns, err.max().item(), err.mean().item())
+        ws.check()

@@ -177,3 +177,32 @@ def test_base_collector_accumulates_over_steps_and_round_trips_its_file(tmp_path
         assert all(t[n].dtype == torch.uint8 and tuple(t[n].shape) == (n_kv, 128) and not t[n].is_cuda for n in ("k3", "k4", "v3", "v4"))
         assert np.array_equal(t["k3"].numpy(), k3) and np.array_equal(t["k4"].numpy(), k4)
         assert np.array_equal(t["v3"].numpy(), v3) and np.array_equal(t["v4"].numpy(), v4)
+
+
+def test_config_0_recipe_equals_the_oracle():
+    """Config 0 as BASELINE.json words it (the reference's own CPU-runnable case, /root/reference/tests/test_codec.py:6-19 and
+    examples/compress_decompress.py:23-26): K [8 kv heads, 4096 tokens, 128] seed 0, element = N(0,1) * sigma_c with sigma_c log-uniform
+    in [2^-4, 2^4], with probability 0.002 per 8-element group one element x 2^12, bases from the first 1024 tokens, encoded as 16-token
+    tiles and decoded.  Bases, every page field, the page size, the tier shares and the decoded rows equal the CPU oracle's."""
+    dev = require_gpu()
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    from bench import make_kv, tier_shares
+    from gaac_amd import Codec, TileEncoder
+    x = make_kv(0, 8, 4096)
+    x16 = to_u16(x)
+    xd = x.to(dev)
+    codec = Codec(8, dev).calibrate(xd[:, :1024])
+    b3, b4 = O.calibrate(x16[:, :1024], 8)
+    assert np.array_equal(codec.base3.cpu().numpy(), b3) and np.array_equal(codec.base4.cpu().numpy(), b4)
+    page = TileEncoder("k", dev).encode(codec, xd)
+    want = O.encode(x16, "k", b3, b4, 8)
+    assert_pages_equal(native_to_reference_page(page), want)
+    n_esc = int(want.ovf_head_start[-1])
+    assert page.nbytes == O.page_nbytes(8, 4096, n_esc) and abs(page.ratio - 8 * 4096 * 256 / page.nbytes) < 1e-12
+    assert 1.39 < page.ratio < 1.42
+    s3, s4, sr = tier_shares(page)
+    tags = np.stack([(want.flags.astype(np.int64) >> (2 * g)) & 3 for g in range(16)], -1)
+    assert abs(s4 - (tags == 1).mean()) < 1e-12 and abs(sr - (tags == 3).mean()) < 1e-12 and 0.85 < s3 < 0.93 and 0.001 < sr < 0.006
+    back = to_u16(Codec.decode(page))
+    assert np.array_equal(back, x16) and np.array_equal(O.decode(want), x16)

@@ -6,7 +6,7 @@ import pytest
 import torch
 
 from oracle import gaac_oracle as O
-from common import kv_like16, to_bf16, to_u16, randn_bf16
+from common import kv_like16, to_bf16, to_u16, randn_bf16, attention_error_bound
 from gpu_util import require_gpu
 
 pytestmark = pytest.mark.gpu
@@ -205,3 +205,50 @@ def test_bad_arguments_raise():
         st.attention(q, buf, bt, sl, nsplit=1, max_seq_len=16 * 3)       # more blocks than the table holds
     with pytest.raises(RuntimeError, match="GQA"):
         st.attention(torch.zeros(1, N_KV * 17, 128, dtype=torch.bfloat16, device=dev), buf, bt, sl, nsplit=1)
+
+
+def test_escape_bytes_at_the_very_end_of_the_pools_last_slot():
+    """The pool is exactly num_blocks * 2 * n_kv slots long (an engine's own block buffer has no slack behind it), and the attention kernel
+    prefetches a lane's escape bytes as one 8-byte load: a tile whose escape bytes fill the slot's 128-byte room to within its last
+    bytes, stored in the LAST slot of the pool (last block, last kv head, V; the K slot before it likewise), must be read without
+    touching a byte behind the pool and decode right.  Lanes whose bytes start in the slot's last 7 bytes take the slow look-up."""
+    dev = require_gpu()
+    from gaac_amd.paged import LayerState, build_store_entries
+    bases = _bases(dev)
+    b = {k: v.cpu().numpy() for k, v in bases.items()}
+    # rows whose last kv head carries, per kind, a tile with 124..128 escape bytes (4-bit and raw groups): a random subset of elements
+    # is scaled by 8, the subset's density searched until the tile's byte count lands there
+    def tile_with_full_slot(kind, seed0):
+        for seed in range(seed0, seed0 + 2000):
+            rng = np.random.default_rng(seed)
+            x = kv_like16(N_KV, 16, seed=seed, outliers=0.0, scale_seed=2000 if kind == "k" else 2001)
+            f = O.bf16_to_f32(x)
+            hit = rng.random(f.shape) < rng.uniform(0.012, 0.03)
+            x = O.f32_to_bf16_rne(np.where(hit, f * 8.0, f).astype(np.float32))
+            tm = O.encode_token_major(x, kind, b[kind + "3"], b[kind + "4"], N_KV)
+            nbytes = int(tm["row_bytes"][N_KV - 1].sum())
+            if 124 <= nbytes <= 128: return x, nbytes
+        raise AssertionError("no candidate tile found")
+    xk, nk = tile_with_full_slot("k", 1000)
+    xv, nv = tile_with_full_slot("v", 3000)
+    num_blocks = 3
+    st = LayerState(num_blocks, N_KV, 16, bases, 128, dev)
+    buf = torch.zeros(LayerState.pool_bytes(num_blocks, N_KV, 128), dtype=torch.uint8, device=dev)
+    assert buf.numel() == num_blocks * 2 * N_KV * 3008
+    k0, v0 = _rows(16, 77)
+    k16 = np.concatenate([k0, _tok16(xk)]); v16 = np.concatenate([v0, _tok16(xv)])      # [32, n_kv, 128]
+    bt_cpu = np.array([[0, num_blocks - 1]], np.int32)
+    st.store(to_bf16(k16, dev), to_bf16(v16, dev), buf, torch.from_numpy(build_store_entries([0], [32], bt_cpu)).to(dev))
+    st.check()
+    mt = st.mt.cpu().numpy()
+    last = (num_blocks - 1) * 2 * N_KV
+    assert mt[last + 2 * N_KV - 1] == last + 2 * N_KV - 1 and mt[last + 2 * N_KV - 2] == last + 2 * N_KV - 2      # compressed in their slots
+    q16 = randn_bf16((1, N_KV * G, 128), seed=5, scale=0.05)
+    bt = torch.from_numpy(bt_cpu).to(dev); sl = torch.tensor([32], dtype=torch.int32, device=dev)
+    for ns in (1, 2):
+        out = O.bf16_to_f32(to_u16(st.attention(to_bf16(q16, dev), buf, bt, sl, ns, max_seq_len=32))).reshape(N_KV * G, 128)
+        ref, tol = attention_error_bound(q16[0], k16, v16, SCALE)
+        assert (np.abs(out - ref) <= tol).all(), (ns, nk, nv)
+    sk = torch.zeros(32, N_KV, 128, dtype=torch.bfloat16, device=dev); sv = torch.zeros_like(sk)
+    st.decode_blocks(buf, torch.tensor([(0, 0, 16), (num_blocks - 1, 16, 16)], dtype=torch.int32, device=dev), sk, sv)
+    assert np.array_equal(to_u16(sk), k16) and np.array_equal(to_u16(sv), v16)

@@ -12,7 +12,7 @@ import numpy as np
 import pytest
 
 from oracle import gaac_oracle as O
-from common import kv_like16
+from common import kv_like16, randn_bf16
 
 GOLD = os.path.join(os.path.dirname(__file__), "golden")
 
@@ -40,6 +40,28 @@ def test_decode_matches_reference_golden(kind):
     out = O.decode(page)
     assert np.array_equal(out, g["decoded"]) and np.array_equal(out, g["x16"])
     assert np.array_equal(O.row_offsets(g["flags"], page.S), g["ovf_off"])
+
+
+@pytest.mark.parametrize("kind", ["k", "v"])
+def test_torch_restatement_of_the_cpu_path_matches_the_golden_pages_and_the_numpy_oracle(kind):
+    """oracle/gaac_oracle_torch.py (the CPU baseline bench.py times): decode_torch on the reference-written golden page gives the golden
+    rows, also when cut into chunks that end inside a tile's run of rows; sdpa_torch equals the oracle's attention."""
+    import torch
+    from oracle.gaac_oracle_torch import decode_torch, sdpa_torch
+    g = np.load(os.path.join(GOLD, f"codec_{kind}.npz"))
+    page = O.OPage(g["sm"], g["codes"], g["flags"], g["ovf_off"], g["ovf"], g["ovf_head_start"], g["tile_off"],
+                   g["base3"], g["base4"], g["x16"].shape[0], g["x16"].shape[1], int(g["n_kv"]), kind)
+    for chunk in (8192, 16, 32):
+        assert np.array_equal(decode_torch(page, chunk).numpy().view(np.uint16), g["decoded"])
+    x = kv_like16(4, 333, seed=17)      # ragged length, all three tiers, per-head pooling h % n_kv
+    b3, b4 = O.calibrate(x, 2)
+    pg = O.encode(x, kind, b3, b4, 2)
+    d = decode_torch(pg, 48)
+    assert np.array_equal(d.numpy().view(np.uint16), x)
+    q16 = randn_bf16((8, 128), seed=5, scale=0.3)
+    want = O.ref_attention(q16, x.transpose(1, 0, 2), x.transpose(1, 0, 2), 128 ** -0.5)
+    got = sdpa_torch(q16, d, d, 128 ** -0.5).numpy()
+    assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max() + 1e-6
 
 
 # ------------------------------------------------------------------------------------------- independent scalar codec

@@ -1,7 +1,8 @@
 """The entry point that allocates nothing (gaac_attn_fused_static: workspace in a device array built into the library) against
 gaac_attn_fused with caller memory, through the C-ABI: same kernel, same arithmetic, so the outputs are equal bit for bit.  Two calls
 in a row, the second with a smaller input (fewer rows, heads, tokens and splits), then the first again; launches beyond the built-in
-workspace are rejected."""
+workspace are rejected.  gaac_static_init resolves the array's address ahead of a capture, gaac_static_flags copies its failure bits
+out, gaac_static_reset re-arms it (by a kernel), and a captured call replays right."""
 import numpy as np
 import pytest
 import torch
@@ -36,6 +37,8 @@ def test_static_workspace_entry_equals_the_caller_memory_entry():
     big = _case(dev, 2, 4, 4, 4096, 16, seed=51, tail=7)
     small = _case(dev, 1, 2, 2, 333, 3, seed=61, tail=0)
     stream = _lib.stream()
+    _lib.call("gaac_static_init")
+    flags = torch.full((1,), 7, dtype=torch.int32, device=dev)
     for common, ws, rows, _keep in (big, small, big, small):
         want = torch.empty(rows, 128, dtype=torch.bfloat16, device=dev); got = torch.full_like(want, float("nan"))
         p = _lib.ptr
@@ -44,7 +47,27 @@ def test_static_workspace_entry_equals_the_caller_memory_entry():
         torch.cuda.synchronize()
         assert torch.isfinite(want.float()).all()
         assert torch.equal(got.view(torch.int16), want.view(torch.int16))
-    # beyond the built-in workspace: 4 x 32 query rows x 32 splits = 4096 > 4032 partial rows
+    _lib.call("gaac_static_flags", _lib.ptr(flags), stream)
+    torch.cuda.synchronize()
+    assert int(flags) == 0
+    # re-arm (epoch words and records back to zero, by a kernel), then a call captured in a graph and replayed
+    _lib.call("gaac_static_reset", stream)
+    common, ws, rows, _keep = small
+    want = torch.empty(rows, 128, dtype=torch.bfloat16, device=dev); got = torch.full_like(want, float("nan"))
+    _lib.call("gaac_attn_fused", *common, _lib.ptr(ws.pm), _lib.ptr(ws.pl), _lib.ptr(ws.pa), _lib.ptr(ws.epoch), _lib.ptr(want), stream)
+    side = torch.cuda.Stream(); side.wait_stream(torch.cuda.current_stream())
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            _lib.call("gaac_attn_fused_static", *common, _lib.ptr(got), _lib.stream())
+    for _ in range(3):
+        got.fill_(float("nan")); torch.cuda.synchronize()
+        g.replay(); torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    _lib.call("gaac_static_flags", _lib.ptr(flags), stream)
+    torch.cuda.synchronize()
+    assert int(flags) == 0
+    # beyond the built-in workspace: 4 x 32 query rows x 32 splits = 4096 > 4000 partial rows
     common, ws, rows, _keep = _case(dev, 4, 8, 4, 512, 32, seed=71, tail=0)
     out = torch.empty(rows, 128, dtype=torch.bfloat16, device=dev)
     with pytest.raises(RuntimeError, match="exceeds"):
