@@ -24,7 +24,7 @@ _SIGNATURES = {
     "gaac_paged_free": [P, c_int, P, P, P],
     "gaac_paged_release": [P, c_int, P, P, P, c_int, P],
     "gaac_paged_decode": [P, c_int, P, P, P, c_int, P, P, c_long, P, P, P, P, c_int, P],
-    "gaac_paged_attn": [P, c_int, P, P, P, c_int, P, c_int, P, c_int, c_int, c_int, c_float, c_int, P, P, P, P, c_int, P, P, P, P, P, P],
+    "gaac_paged_attn": [P, c_int, P, P, P, c_int, P, c_int, P, c_int, c_int, c_int, c_float, c_int, P, P, P, P, c_int, P, P, P, P, P, P, c_int, P, P, P],
     "gaac_bf16_attn": [P, P, c_int, P, c_long, P, c_int, c_int, c_int, c_float, c_int, P, P, P, P, P, P],
     "gaac_attn_fused": [P] * 16 + [P, P, c_int, c_int, c_int, P, c_int, c_float, c_int, c_int, P, P, P, c_int, c_int, P, P, P, P, P, P],
     "gaac_attn_fused_static": [P] * 16 + [P, P, c_int, c_int, c_int, P, c_int, c_float, c_int, c_int, P, P, P, c_int, c_int, P, P],

@@ -41,6 +41,8 @@ struct AttnArgs {
   // paged slot pool (k_attn_split<true>): sl = tokens per batch row, bt = block table [B][bt_stride], mt = mode table, pool = tile
   // slots of TS bytes, raw = side pool of BF16 tiles; physical tile = block*2*n_kv + 2*kvh + kind
   const uint8_t* pool; const u16* raw; const int* mt; const int* bt; int bt_stride; int TS;
+  // paged: raw tiles queued by the preceding store (gaac_paged_store's freeq) that this launch pushes back onto the free stack (or null)
+  const int* freeq; int n_free; int* stack; int* top;
 #ifdef GAAC_PHASE_TIMING
   long long* dbg;
 #endif
@@ -606,7 +608,7 @@ __device__ __forceinline__ void unit_x_words(const KindRegs& R, const AttnLds& L
     x[u] = L.xlut[(eb4 >> (8 * u)) & 0xFFu];
     bw[u] = tab[(KIND == KIND_K ? u : 0) + NG * ((tag8 >> (2 * u)) & 1u)];
   }
-  if (__builtin_amdgcn_ballot_w64((tag8 & 0xAAu) != 0u || (SLOW && tag8 != 0u && R.pos0 > lim))) {
+  if (__builtin_amdgcn_ballot_w64((tag8 & 0xAAu) != 0u || (SLOW && R.pos0 > lim))) {
     const u64 e64 = (u64)R.e[0] | ((u64)R.e[1] << 32);
 #pragma unroll
     for (int u = 0; u < 4; ++u) {
@@ -648,7 +650,7 @@ __device__ __forceinline__ void consume(const TileRegs& R, WaveState& st, const 
   const u32 kr = R.k.f & 0xAAu, vr = R.v.f & 0xAAu;
   const u32 lim = PAGED ? (u32)(B.TS - SLOT_OV - 8) : 0xFFFFFFFFu;      // paged pool: the 8 prefetched bytes were taken from no further than this
   bool slow = ((kr & (kr - 1u)) | (vr & (vr - 1u))) != 0u;
-  if (PAGED) slow |= (R.k.f != 0u && R.k.pos0 > lim) || (R.v.f != 0u && R.v.pos0 > lim);
+  if (PAGED) slow |= max(R.k.pos0, R.v.pos0) > lim;      // (also lanes without escape bytes: a position that far into a slot is rare)
   if (__builtin_expect(__builtin_amdgcn_ballot_w64(slow) != 0, 0)) {
     unit_x_words<KIND_K, true>(R.k, L, PAGED ? esc_of_tile<PAGED>(B.kov, kto, B.TS) : B.kov, lim, a, q, xk, bk);
     unit_x_words<KIND_V, true>(R.v, L, PAGED ? esc_of_tile<PAGED>(B.vov, vto, B.TS) : B.vov, lim, a, q, xv, bv);
@@ -745,6 +747,13 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
                  "s"(A.k.head_start), "s"(A.k.base3), "s"(A.k.base4), "s"(A.v.sm), "s"(A.v.cd), "s"(A.v.flags), "s"(A.v.tile_off),
                  "s"(A.v.ovf), "s"(A.v.head_start), "s"(A.v.base3), "s"(A.v.base4), "s"(A.kt), "s"(A.tl), "s"(A.nsplit), "s"(A.n_kv),
                  "s"(A.n_q), "s"(A.G), "s"(A.NB), "s"(A.S_pad), "s"(A.tcap));
+  // Paged pool: the launch can take the place of gaac_paged_free (it pops nothing, so pushes are safe here): the grid's last block, the
+  // one with the least to do, pushes the queued raw tiles back before its own work.  The wait keeps the stores' bookkeeping out of
+  // the code every block runs.
+  if (PAGED && A.freeq != nullptr && blockIdx.x == gridDim.x - 1) {
+    for (int i = tid; i < A.n_free; i += NT) { const int r = A.freeq[i]; if (r >= 0) A.stack[atomicAdd(A.top, 1)] = r; }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  }
   // Paged pool: the split index is rotated by the head index: the last split of a sequence carries the raw tile that is still filling,
   // and with equal split counts all of them would otherwise sit on the same XCD, which then finishes long after the others.
   const int bh = (int)blockIdx.x / A.nsplit, split = ((int)blockIdx.x + (PAGED ? bh : 0)) % A.nsplit;
@@ -1238,6 +1247,7 @@ static int attn_split_impl(
   A.epochs = epoch; A.out = (u16*)out;
   GAAC_REQUIRE(!epoch || out, "gaac_attn: the fused merge needs an output buffer");
   A.pool = nullptr; A.raw = nullptr; A.mt = nullptr; A.bt = nullptr; A.bt_stride = 0; A.TS = 0;
+  A.freeq = nullptr; A.n_free = 0; A.stack = nullptr; A.top = nullptr;
 #ifdef GAAC_PHASE_TIMING
   A.dbg = g_dbg;
 #endif
@@ -1401,8 +1411,10 @@ extern "C" int gaac_paged_attn(
     const uint8_t* pool, int TS, const void* raw, const int* mt, const int* bt, int bt_stride, const int* seq_lens, int max_seq_len,
     const void* q, int B, int n_q, int n_kv, float scale, int nsplit,
     const uint8_t* b3k, const uint8_t* b4k, const uint8_t* b3v, const uint8_t* b4v, int NB,
-    unsigned long long* pm, unsigned long long* pl, unsigned long long* pa, unsigned int* epoch, void* out, void* stream) {
+    unsigned long long* pm, unsigned long long* pl, unsigned long long* pa, unsigned int* epoch, void* out,
+    const int* freeq, int n_free, int* stack, int* top, void* stream) {
   GAAC_REQUIRE(n_kv > 0 && n_q > 0 && n_q % n_kv == 0 && n_q / n_kv <= GMAX, "GQA group size must be 1..%d (n_q=%d, n_kv=%d)", GMAX, n_q, n_kv);
+  GAAC_REQUIRE(!freeq || (n_free > 0 && stack && top), "gaac_paged_attn: a free queue needs its length, the stack and its top");
   GAAC_REQUIRE(pool && raw && mt && bt && seq_lens && q && b3k && b4k && b3v && b4v && pm && pl && pa && epoch && out, "gaac_paged_attn: null pointer");
   GAAC_REQUIRE(B > 0 && NB > 0 && TS >= SLOT_OV + 16 && TS % 16 == 0 && bt_stride > 0, "gaac_paged_attn: bad sizes B=%d NB=%d TS=%d (a slot is %d bytes plus at least 16 for escapes)", B, NB, TS, SLOT_OV);
   GAAC_REQUIRE(nsplit >= 1 && nsplit <= MAX_SLOTS, "gaac_paged_attn: nsplit must be in 1..%d", MAX_SLOTS);
@@ -1417,6 +1429,7 @@ extern "C" int gaac_paged_attn(
   A.kt = nullptr; A.vt = nullptr; A.tl = nullptr; A.tcap = 0;
   A.epochs = epoch; A.out = (u16*)out;
   A.pool = pool; A.raw = (const u16*)raw; A.mt = mt; A.bt = bt; A.bt_stride = bt_stride; A.TS = TS;
+  A.freeq = freeq; A.n_free = freeq ? n_free : 0; A.stack = stack; A.top = top;
 #ifdef GAAC_PHASE_TIMING
   A.dbg = g_dbg;
 #endif

@@ -58,6 +58,7 @@ class LayerState:
         self.err = torch.zeros(1, **i32)
         self.b3k, self.b4k, self.b3v, self.b4v = (bases[k].to(device).to(torch.uint8).reshape(n_kv, D).contiguous() for k in ("k3", "k4", "v3", "v4"))
         self._ws = {}
+        self._pending_free = None      # (freeq, n): raw tiles a store queued and no launch has pushed back yet
 
     @staticmethod
     def pool_bytes(num_blocks: int, n_kv: int, ovf_slot: int = 128) -> int:
@@ -71,9 +72,19 @@ class LayerState:
     def _base_ptrs(self):
         return tuple(_lib.ptr(t) for t in self.bases)
 
-    def store(self, key: torch.Tensor, value: torch.Tensor, buf: torch.Tensor, ent: torch.Tensor, freeq: torch.Tensor | None = None):
+    def _flush_free(self):
+        if self._pending_free is not None:
+            freeq, n = self._pending_free
+            self._pending_free = None
+            _lib.call("gaac_paged_free", _lib.ptr(freeq), n, _lib.ptr(self.stack), _lib.ptr(self.top), _lib.stream())
+
+    def store(self, key: torch.Tensor, value: torch.Tensor, buf: torch.Tensor, ent: torch.Tensor, freeq: torch.Tensor | None = None,
+              defer_free: bool = False):
         """key/value: [num_tokens, n_kv, D] bf16 (or int16 views); buf: uint8 flat block pool; ent: int32 [E,4] = (blk, tok0, off0, n);
-        freeq: int32 [E*2*n_kv] scratch (allocated when omitted)."""
+        freeq: int32 [E*2*n_kv] scratch (allocated when omitted).  defer_free: the raw tiles this store gives back are pushed onto
+        the free stack by the next attention() launch of this layer instead of a launch of their own (a decode step is then two
+        launches); any other call that needs the stack first (another store, release_blocks, check) pushes them itself."""
+        self._flush_free()
         E = ent.shape[0]
         if E == 0: return
         if key.stride(-1) != 1 or key.stride(1) != D or value.stride(-1) != 1 or value.stride(1) != D:
@@ -83,7 +94,8 @@ class LayerState:
         p = _lib.ptr
         _lib.call("gaac_paged_store", p(key), p(value), key.stride(0), value.stride(0), p(ent), E, p(buf), self.TS, p(self.raw), p(self.mt),
                   p(self.stack), p(self.top), p(self.err), p(freeq), *self._base_ptrs(), self.n_kv, _lib.stream())
-        _lib.call("gaac_paged_free", p(freeq), n, p(self.stack), p(self.top), _lib.stream())
+        self._pending_free = (freeq, n)
+        if not defer_free: self._flush_free()
 
     def decode_blocks(self, buf: torch.Tensor, pairs: torch.Tensor, sk: torch.Tensor, sv: torch.Tensor):
         """pairs: int32 [P,3] (block, first scratch row, valid rows); sk/sv: flat K/V [rows, n_kv, D] bf16 (written)."""
@@ -99,11 +111,13 @@ class LayerState:
         """blocks: int32 [F] block ids whose content is dead."""
         F = blocks.shape[0]
         if F == 0: return
+        self._flush_free()
         p = _lib.ptr
         _lib.call("gaac_paged_release", p(blocks), F, p(self.mt), p(self.stack), p(self.top), self.n_kv, _lib.stream())
 
     def check(self):
         """Host poll (every 16 steps in the reference, backend.py:233-236): raises when the raw side pool ran dry."""
+        self._flush_free()
         for ws in self._ws.values(): ws.check()      # a fused attention launch that gave up a wait: re-arm with ws.reset()
         failed = int(self.err)
         if failed:
@@ -115,14 +129,17 @@ class LayerState:
         if out is None: out = torch.empty(B, n_q * D, dtype=q.dtype, device=q.device)
         ws = self._ws.get((B, n_q, nsplit))
         if ws is None: ws = self._ws[(B, n_q, nsplit)] = AttnWorkspace(B * n_q, nsplit, q.dtype, q.device, with_out=False)
-        return paged_attention(q, out, buf, self.raw, self.mt, bt, seq_lens, self.bases, self.TS, n_q, self.n_kv, nsplit, max_seq_len, ws)
+        free, self._pending_free = self._pending_free, None
+        return paged_attention(q, out, buf, self.raw, self.mt, bt, seq_lens, self.bases, self.TS, n_q, self.n_kv, nsplit, max_seq_len, ws,
+                               free=None if free is None else (free[0], free[1], self.stack, self.top))
 
 
-def paged_attention(q, out, buf, raw, mt, bt, seq_lens, bases, TS, n_q, n_kv, nsplit, max_seq_len=None, ws=None):
+def paged_attention(q, out, buf, raw, mt, bt, seq_lens, bases, TS, n_q, n_kv, nsplit, max_seq_len=None, ws=None, free=None):
     """q: [B, n_q, 128] bf16 contiguous; out: [B, n_q*128] bf16 (written); buf: uint8 flat block pool; raw: [tiles,16,128] bf16;
     mt: int32 [num_blocks*2*n_kv]; bt: int32 [B, max_blocks]; seq_lens: int32 [B]; bases: (b3k,b4k,b3v,b4v) uint8 [n_kv,128].
     max_seq_len: host-side bound of seq_lens (default: what the block table can address).  ws: the launch's
-    AttnWorkspace (default: one cached per device, stream and launch shape, so repeated calls allocate nothing)."""
+    AttnWorkspace (default: one cached per device, stream and launch shape, so repeated calls allocate nothing).  free: (freeq, n, stack,
+    top) of a preceding store whose raw tiles this launch pushes back (LayerState.store(defer_free=True))."""
     B = q.shape[0]
     if q.shape[-1] != D: raise RuntimeError("head_dim must be 128")
     if max_seq_len is None: max_seq_len = bt.shape[1] * BLOCK
@@ -132,5 +149,6 @@ def paged_attention(q, out, buf, raw, mt, bt, seq_lens, bases, TS, n_q, n_kv, ns
     q = q.contiguous()
     _lib.call("gaac_paged_attn", p(buf), TS, p(raw), p(mt), p(bt), bt.stride(0), p(seq_lens), int(max_seq_len), p(q), B, n_q, n_kv,
               float(1.0 / (D ** 0.5)), nsplit, p(bases[0]), p(bases[1]), p(bases[2]), p(bases[3]), bases[0].shape[0],
-              p(ws.pm), p(ws.pl), p(ws.pa), p(ws.epoch), p(out), _lib.stream())
+              p(ws.pm), p(ws.pl), p(ws.pa), p(ws.epoch), p(out),
+              *((p(free[0]), int(free[1]), p(free[2]), p(free[3])) if free is not None else (None, 0, None, None)), _lib.stream())
     return out

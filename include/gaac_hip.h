@@ -159,12 +159,15 @@ int gaac_paged_decode(const uint8_t* pool, int TS, const void* raw, const int* m
  * bt int32 [B][bt_stride] and the mode table; seq_lens int32 [B] (tokens incl. the filling block; no separate tail); max_seq_len =
  * an upper bound of seq_lens known to the host (checked against the block table's width).  Any nsplit >= 1 works for any length (a
  * block resolves 1024 tiles of its split at a time).  Partial records pm, pl [B*n_q*nsplit], pa [B*n_q*nsplit*128] and the epoch
- * buffer [2 + B*n_kv*nsplit] as in gaac_attn_fused; out bf16 [B*n_q][128]. */
+ * buffer [2 + B*n_kv*nsplit] as in gaac_attn_fused; out bf16 [B*n_q][128].
+ * freeq != NULL: the launch also does the work of gaac_paged_free(freeq, n_free, stack, top) for the queue the preceding
+ * gaac_paged_store filled (the attention pops nothing, so pushes cannot race a pop here): a decode step is then two launches
+ * instead of the reference's three (store.py:108-114 is a launch of its own). */
 int gaac_paged_attn(const uint8_t* pool, int TS, const void* raw, const int* mt, const int* bt, int bt_stride, const int* seq_lens,
                     int max_seq_len, const void* q, int B, int n_q, int n_kv, float scale, int nsplit,
                     const uint8_t* b3k, const uint8_t* b4k, const uint8_t* b3v, const uint8_t* b4v, int NB,
                     unsigned long long* pm, unsigned long long* pl, unsigned long long* pa, unsigned int* epoch, void* out,
-                    void* stream);
+                    const int* freeq, int n_free, int* stack, int* top, void* stream);
 
 /* Baseline, not part of the compressed path: decode attention over UNCOMPRESSED bf16 K/V [B*n_kv][head_stride_tokens][128] (S tokens
  * per head, or seq_lens[b] <= S tokens for batch row b when seq_lens != NULL) with the same block / wave / MFMA structure, merge and

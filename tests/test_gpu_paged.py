@@ -252,3 +252,48 @@ def test_escape_bytes_at_the_very_end_of_the_pools_last_slot():
     sk = torch.zeros(32, N_KV, 128, dtype=torch.bfloat16, device=dev); sv = torch.zeros_like(sk)
     st.decode_blocks(buf, torch.tensor([(0, 0, 16), (num_blocks - 1, 16, 16)], dtype=torch.int32, device=dev), sk, sv)
     assert np.array_equal(to_u16(sk), k16) and np.array_equal(to_u16(sv), v16)
+
+
+def test_attention_launch_that_also_frees_equals_the_separate_free_launch():
+    """LayerState.store(defer_free=True) leaves the raw tiles it gives back to the next attention launch (two launches per decode step
+    instead of three).  Two pools go through the same prompts and 40 decode steps, one with the separate free launch, one deferring: after
+    every step the same tiles are compressed or raw, the number of free tiles is the same and no raw tile is lost or handed out twice, the
+    attention outputs are equal bit for bit, and a store that follows a deferred store without an attention in between pushes the queue itself."""
+    dev = require_gpu()
+    from gaac_amd.paged import build_store_entries
+    pools = [_Pool(dev, n_seq=3, max_blocks=12, num_blocks=40, raw_tiles=40, seed=4) for _ in range(2)]
+    def step(P, new, defer):
+        seqs = sorted(new)
+        ent = build_store_entries([P.lens[s] for s in seqs], [len(new[s][0]) for s in seqs], [P.bt_cpu[s] for s in seqs])
+        k = to_bf16(np.concatenate([new[s][0] for s in seqs]), dev); v = to_bf16(np.concatenate([new[s][1] for s in seqs]), dev)
+        P.st.store(k, v, P.buf, torch.from_numpy(ent).to(dev), defer_free=defer)
+        for s in seqs:
+            P.hist[s] = (np.concatenate([P.hist[s][0], new[s][0]]), np.concatenate([P.hist[s][1], new[s][1]]))
+            P.lens[s] += len(new[s][0])
+    def attend(P, q16):
+        sl = torch.tensor(P.lens, dtype=torch.int32, device=dev)
+        return to_u16(P.st.attention(to_bf16(q16, dev), P.buf, P.bt, sl, 2, max_seq_len=max(P.lens)))
+    def same_state():
+        a, b = pools
+        ta, tb = int(a.st.top), int(b.st.top)
+        ma, mb = a.st.mt.cpu().numpy(), b.st.mt.cpu().numpy()
+        # the same tiles are compressed in place / raw (which raw tile a slot got depends on the order of the pushes)
+        assert ta == tb and np.array_equal(ma >= 0, mb >= 0) and np.array_equal(ma[ma >= 0], mb[mb >= 0])
+        for P, m, t in ((a, ma, ta), (b, mb, tb)):      # every raw tile is either in use exactly once or on the free stack exactly once
+            assert sorted((~m[m < 0]).tolist() + P.st.stack[:t].tolist()) == list(range(P.st.raw.shape[0]))
+    prompts = {0: _rows(30, 1), 1: _rows(47, 2), 2: _rows(15, 3)}
+    for P, d in zip(pools, (False, True)): step(P, prompts, d)
+    for P, d in zip(pools, (False, True)): step(P, {2: _rows(1, 4)}, d)      # sequence 2's block fills up; a second store in a row
+    q16 = randn_bf16((3, N_KV * G, 128), seed=8, scale=0.1)
+    assert np.array_equal(attend(pools[0], q16), attend(pools[1], q16))
+    same_state()
+    for t in range(40):
+        new = {s: _rows(1, 100 + 3 * t + s) for s in range(3)}
+        for P, d in zip(pools, (False, True)): step(P, new, d)
+        assert pools[1].st._pending_free is not None and pools[0].st._pending_free is None
+        q16 = randn_bf16((3, N_KV * G, 128), seed=300 + t, scale=0.1)
+        assert np.array_equal(attend(pools[0], q16), attend(pools[1], q16))
+        assert pools[1].st._pending_free is None
+        same_state()
+    pools[1].check([0, 1, 2], randn_bf16((3, N_KV * G, 128), seed=9, scale=0.1))
+    for P in pools: P.st.check()
