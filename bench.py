@@ -55,7 +55,12 @@ def clone_store(page):
     return c
 
 
-_CPU_PAGES = None      # per-head oracle pages of the CPU baseline, inherited by its forked workers
+_CPU_PAGES = None      # per-head oracle pages of the CPU baseline (set in each worker process by _cpu_worker_init)
+
+
+def _cpu_worker_init(pages):
+    global _CPU_PAGES
+    _CPU_PAGES = pages
 
 
 def _cpu_head_pass(h: int):
@@ -71,9 +76,10 @@ def _cpu_head_pass(h: int):
 
 def cpu_baseline(k16: np.ndarray, v16: np.ndarray, q16: np.ndarray, b3k, b4k, b3v, b4v, scale: float, heads: int, n_kv: int, g: int) -> dict:
     """The reference's CPU path (decompress both pages + fp32 SDPA) on `heads` kv heads of the same workload (bounded sample), timed on
-    this box's host cores.  Must be called BEFORE the process touches the GPU: it forks worker processes.
+    this box's host cores.  Called before the process touches the GPU; the worker processes are spawned (fresh interpreters that
+    inherit nothing of this one's runtime state, and never use the GPU) and joined before it returns.
     (a) torch ops on torch's intra-op threads (oracle/gaac_oracle_torch.py, the form the reference's own CPU path has): `value`;
-    (b) the numpy oracle on one thread and with one forked worker per kv head, for comparison.
+    (b) the numpy oracle on one thread and with one worker process per kv head, for comparison.
     Pages are encoded beforehand by the oracle (not timed).  Every pass is checked: decoded rows equal the input bit for bit."""
     global _CPU_PAGES
     import multiprocessing as mp
@@ -102,7 +108,7 @@ def cpu_baseline(k16: np.ndarray, v16: np.ndarray, q16: np.ndarray, b3k, b4k, b3
     dt1 = time.perf_counter() - t0
     assert res == [(True, w) for w in want]
     workers = max(1, min(heads, len(os.sched_getaffinity(0)), 16))
-    pool = mp.get_context("fork").Pool(workers)
+    pool = mp.get_context("spawn").Pool(workers, initializer=_cpu_worker_init, initargs=(_CPU_PAGES,))
     try:
         pool.map(_cpu_head_pass, range(heads))      # warm-up: workers started, pages touched
         t0 = time.perf_counter()
@@ -117,7 +123,7 @@ def cpu_baseline(k16: np.ndarray, v16: np.ndarray, q16: np.ndarray, b3k, b4k, b3
             "what": "the reference's CPU path restated: decompress K and V pages + fp32 scaled_dot_product_attention, PyTorch ops on the host (oracle/gaac_oracle_torch.py)",
             "numpy_port_one_thread_us_per_layer": round(dt1 * 1e6 * up, 1), "numpy_port_workers_us_per_layer": round(dtn * 1e6 * up, 1), "numpy_port_workers": workers,
             "sample": f"{heads} of {n_kv} kv heads x {k16.shape[1]} tokens (K and V); torch ops: mean of {reps_t} passes, {dt_t:.2f} s on {threads} torch threads; "
-                      f"numpy oracle: one pass each, {dt1:.2f} s on 1 thread, {dtn:.2f} s with {workers} forked workers (one kv head each); scaled x{up:g}; "
+                      f"numpy oracle: one pass each, {dt1:.2f} s on 1 thread, {dtn:.2f} s with {workers} worker processes (one kv head each); scaled x{up:g}; "
                       f"host offers {len(os.sched_getaffinity(0))} cpus; run before the process initialised the GPU"}
 
 
@@ -156,7 +162,7 @@ def main():
     if a.gpus != 1:
         print("bench.py measures one MI355X; this build has no multi-GPU path (the hot path shards by kv head without any exchange). Use --gpus 1.", file=sys.stderr)
         sys.exit(2)
-    if torch.cuda.device_count() == 0:      # (counting devices does not initialise the GPU: the CPU baseline below forks workers first)
+    if torch.cuda.device_count() == 0:      # (counting devices does not initialise the GPU: the CPU baseline below runs first)
         print("bench.py needs a GPU: the product has no CPU path.", file=sys.stderr); sys.exit(2)
     global N_KV, G
     v_range = (-4.0, 4.0)
@@ -173,7 +179,7 @@ def main():
     # ---- synthetic inputs (config 1): K seed 1, V seed 2, q seed 3; bases from the first 1024 tokens
     k_all, v_all = make_kv(1, H, S_CTX + TAIL_TOK), make_kv(2, H, S_CTX + TAIL_TOK, *v_range)
     q = torch.randn(B, n_q, D, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16)
-    # ---- the CPU baseline runs first, while this process has not touched the GPU (it forks worker processes); its bases come from the
+    # ---- the CPU baseline runs first, while this process has not touched the GPU (it starts and joins worker processes); its bases come from the
     # oracle's own calibration and are compared with the HIP calibration below
     cpu_res, cpu_bases = None, None
     if a.cpu_heads > 0 and B == 1 and not a.kernel_only:
