@@ -23,7 +23,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the attention kernel on the default workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by the
 # library's plain 64 MiB copy kernel (factors 1.99937 read, 1.0 write); the profiler runs are separate from a timing run, so the
 # figure is carried here and reported only for the configuration it was measured on.
-MEASURED_TRAFFIC = {"nsplit": 32, "bytes": 196042051,
+MEASURED_TRAFFIC = {"nsplit": 32, "bytes": 196012470,
                     "source": "constant in bench.py, not measured by this run: profiles/k_attn_split_config1_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE)"}
 
 

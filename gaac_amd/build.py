@@ -9,6 +9,7 @@ import os, subprocess, sys, shutil
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libgaac_hip.so")
+LIB_W12 = os.path.join(HERE, "libgaac_hip_w12.so")            # measurement build -DGAAC_WAVES12: twelve-wave blocks, three waves per SIMD (see attn.hip); on demand only
 LIB_TIMING = os.path.join(HERE, "libgaac_hip_timing.so")      # same sources with -DGAAC_PHASE_TIMING (per-block phase time stamps); built on demand only
 SOURCES = ["codec.hip", "attn.hip", "cache.hip", "paged.hip"]
 # bench.py's measurement aids (read probe, plain copy): their own library next to bench.py, not in the product library
@@ -24,13 +25,15 @@ FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
 SOURCE_FLAGS = {"attn.hip": ["-mllvm", "-amdgpu-sched-strategy=max-ilp"]}
 
 
-def build(verbose: bool = True, extra_flags: list[str] | None = None, timing: bool = False) -> str:
-    """timing=True builds the instrumented variant (libgaac_hip_timing.so, loaded through the GAAC_HIP_LIB override)."""
+def build(verbose: bool = True, extra_flags: list[str] | None = None, timing: bool = False, waves12: bool = False) -> str:
+    """timing=True builds the instrumented variant (libgaac_hip_timing.so), waves12=True the twelve-wave measurement build
+    (libgaac_hip_w12.so); both are loaded through the GAAC_HIP_LIB override and neither is part of the product."""
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     objs = []
     if timing: extra_flags = [*(extra_flags or []), "-DGAAC_PHASE_TIMING"]
+    if waves12: extra_flags = [*(extra_flags or []), "-DGAAC_WAVES12"]
     for src in SOURCES:
-        obj = os.path.join(CSRC, src.replace(".hip", ".timing.o" if timing else ".o"))
+        obj = os.path.join(CSRC, src.replace(".hip", ".timing.o" if timing else ".w12.o" if waves12 else ".o"))
         cmd = [hipcc, *FLAGS, *SOURCE_FLAGS.get(src, []), *(extra_flags or []), "-c", os.path.join(CSRC, src), "-o", obj]
         if verbose: print(" ".join(cmd), flush=True)
         r = subprocess.run(cmd, capture_output=True, text=True)
@@ -39,7 +42,7 @@ def build(verbose: bool = True, extra_flags: list[str] | None = None, timing: bo
             raise RuntimeError(f"hipcc failed on {src}:\n{err}")
         if verbose and err.strip(): print(err, file=sys.stderr)
         objs.append(obj)
-    out = LIB_TIMING if timing else LIB
+    out = LIB_TIMING if timing else LIB_W12 if waves12 else LIB
     cmd = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", out]
     if verbose: print(" ".join(cmd), flush=True)
     r = subprocess.run(cmd, capture_output=True, text=True)
@@ -63,3 +66,4 @@ if __name__ == "__main__":
     print(build())
     print(build_bench_lib())
     if "--timing" in sys.argv: print(build(timing=True))
+    if "--waves12" in sys.argv: print(build(waves12=True))

@@ -21,6 +21,17 @@
 #include "gaac_capi.h"
 #include "../../include/gaac_hip.h"
 
+// GAAC_WAVES12 (python -m gaac_amd.build --waves12 -> libgaac_hip_w12.so) is a measurement build, not the product: launches of up to
+// 256 blocks over contiguous stores with host lengths run twelve-wave blocks, three waves per SIMD instead of two.  The register cap
+// falls from 256 to 168 per lane; to get under it without spilling the tile loop, this build reads the query words from LDS for every
+// score product instead of keeping them in 16 registers, and looks up the V side's escape and base words after the score products
+// instead of together with the K side's.  Both cost time at two waves per SIMD, which is why the product does neither.
+#ifdef GAAC_WAVES12
+constexpr bool WAVES12 = true;
+#else
+constexpr bool WAVES12 = false;
+#endif
+
 namespace gaac {
 
 constexpr int GMAX = 16;         // query heads per kv head the MFMA tile can carry
@@ -219,9 +230,11 @@ constexpr int EPOCH_WORDS = 2;      // words of the epoch buffer ahead of the ar
 __device__ __forceinline__ void mark_arrival(const AttnArgs& A, u32 epoch) {
   __hip_atomic_store(A.epochs + EPOCH_WORDS + blockIdx.x, epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-template <int NW>
-__device__ __forceinline__ void merge_heads(const AttnArgs& A, long qh0, int G, u32 epoch, int rank, int mergers, int tid, MergeScratch<NW>& X) {
+template <int NWB>      // NWB: waves of the block; twelve-wave blocks (measurement build) merge with their first eight waves
+__device__ __forceinline__ void merge_heads(const AttnArgs& A, long qh0, int G, u32 epoch, int rank, int mergers, int tid, MergeScratch<(NWB > 8 ? 8 : NWB)>& X) {
+  constexpr int NW = NWB > 8 ? 8 : NWB;
   const int wave = tid >> 6, lane = tid & 63;
+  if (NWB > NW && wave >= NW) { if (blockIdx.x == gridDim.x - 1) lds_barrier(); return; }      // (the last block meets once more below)
   const bool last = blockIdx.x == gridDim.x - 1;
   // The last block of the grid advances the epoch word for the next launch, once every block of this launch has marked its arrival
   // (and so has read the word).  The marks' first read is issued here, ahead of the merge work, and looked at after it: by then the
@@ -651,12 +664,13 @@ __device__ __forceinline__ void consume(const TileRegs& R, WaveState& st, const 
   const u32 lim = PAGED ? (u32)(B.TS - SLOT_OV - 8) : 0xFFFFFFFFu;      // paged pool: the 8 prefetched bytes were taken from no further than this
   bool slow = ((kr & (kr - 1u)) | (vr & (vr - 1u))) != 0u;
   if (PAGED) slow |= max(R.k.pos0, R.v.pos0) > lim;      // (also lanes without escape bytes: a position that far into a slot is rare)
-  if (__builtin_expect(__builtin_amdgcn_ballot_w64(slow) != 0, 0)) {
+  const bool any_slow = __builtin_amdgcn_ballot_w64(slow) != 0;
+  if (__builtin_expect(any_slow, 0)) {
     unit_x_words<KIND_K, true>(R.k, L, PAGED ? esc_of_tile<PAGED>(B.kov, kto, B.TS) : B.kov, lim, a, q, xk, bk);
-    unit_x_words<KIND_V, true>(R.v, L, PAGED ? esc_of_tile<PAGED>(B.vov, vto, B.TS) : B.vov, lim, a, q, xv, bv);
+    if (!WAVES12) unit_x_words<KIND_V, true>(R.v, L, PAGED ? esc_of_tile<PAGED>(B.vov, vto, B.TS) : B.vov, lim, a, q, xv, bv);
   } else {
     unit_x_words<KIND_K, false>(R.k, L, nullptr, lim, a, q, xk, bk);
-    unit_x_words<KIND_V, false>(R.v, L, nullptr, lim, a, q, xv, bv);
+    if (!WAVES12) unit_x_words<KIND_V, false>(R.v, L, nullptr, lim, a, q, xv, bv);
   }
   // ---- scores: S[tok 4q+r][head a]
   f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
@@ -666,7 +680,12 @@ __device__ __forceinline__ void consume(const TileRegs& R, WaveState& st, const 
     unit_sm(R.k.pay, u, slo, shi);
     decode_unit_x(slo, shi, unit_code_word(R.k.pay.c0, R.k.pay.c1, R.k.pay.c2, u), xk[u], bk[u], w);
     const u32x4 av = {w[0], w[1], w[2], w[3]};
-    sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av), __builtin_bit_cast(bf16x8, qf[u]), sacc, 0, 0, 0);
+    const u32x4 qu = WAVES12 ? L.qw[a][4 * q + u] : qf[u];
+    sacc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, av), __builtin_bit_cast(bf16x8, qu), sacc, 0, 0, 0);
+  }
+  if (WAVES12) {      // measurement build: the V side's look-ups only now, when the K side's registers are free
+    if (__builtin_expect(any_slow, 0)) unit_x_words<KIND_V, true>(R.v, L, PAGED ? esc_of_tile<PAGED>(B.vov, vto, B.TS) : B.vov, lim, a, q, xv, bv);
+    else unit_x_words<KIND_V, false>(R.v, L, nullptr, lim, a, q, xv, bv);
   }
   // ---- online softmax per head a over the tile's 16 tokens (4 in this lane, 4 quads); exp2(score * scale*log2e - mu)
   const int tok0 = tile * T + 4 * q;
@@ -1025,7 +1044,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) k_attn_split(const A
   GAAC_STAMP(4);
   if (fused && rank >= 0 && A.nslot > 1) {
     lds_barrier();      // every thread is done with the block-merge buffer, which becomes the mergers' scratch
-    merge_heads<NW>(A, qh0, G, epoch, rank, mergers, tid, *reinterpret_cast<MergeScratch<NW>*>(&M.acc[0][0][0]));
+    merge_heads<NW>(A, qh0, G, epoch, rank, mergers, tid, *reinterpret_cast<MergeScratch<(NW > 8 ? 8 : NW)>*>(&M.acc[0][0][0]));
   }
   GAAC_STAMP(5);
 }
@@ -1254,7 +1273,11 @@ static int attn_split_impl(
   // few blocks: one 8-wave block per CU (half as many partials); otherwise two 4-wave blocks per CU
   const bool wide = (long)B * n_kv * nslot <= 256;
   const dim3 grid(B * n_kv * nslot), block(wide ? 512 : 256);
+#ifdef GAAC_WAVES12
+  if (wide && S_all >= 0) hipLaunchKernelGGL((k_attn_split<false, 12, true>), grid, dim3(768), 0, (hipStream_t)stream, A);
+#else
   if (wide && S_all >= 0) hipLaunchKernelGGL((k_attn_split<false, 8, true>), grid, block, 0, (hipStream_t)stream, A);
+#endif
   else if (wide) hipLaunchKernelGGL((k_attn_split<false, 8, false>), grid, block, 0, (hipStream_t)stream, A);
   else if (S_all >= 0) hipLaunchKernelGGL((k_attn_split<false, 4, true>), grid, block, 0, (hipStream_t)stream, A);
   else hipLaunchKernelGGL((k_attn_split<false, 4, false>), grid, block, 0, (hipStream_t)stream, A);
