@@ -62,8 +62,9 @@ def build_bench_lib(verbose: bool = True) -> str:
     return BENCH_LIB
 
 
-if __name__ == "__main__":
-    print(build())
-    print(build_bench_lib())
+if __name__ == "__main__":      # no option: the library and bench.py's kernels; --timing / --waves12: only that measurement build
     if "--timing" in sys.argv: print(build(timing=True))
     if "--waves12" in sys.argv: print(build(waves12=True))
+    if "--timing" not in sys.argv and "--waves12" not in sys.argv:
+        print(build())
+        print(build_bench_lib())
