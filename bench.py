@@ -141,6 +141,7 @@ def bench_lib():
         P = ctypes.c_void_p
         lib.gaac_stream_copy.argtypes = [P, P, ctypes.c_long, P]; lib.gaac_stream_copy.restype = ctypes.c_int
         lib.gaac_read_probe.argtypes = [P] * 12 + [ctypes.c_int] * 5 + [P, P]; lib.gaac_read_probe.restype = ctypes.c_int
+        lib.gaac_read_probe_paged.argtypes = [P, ctypes.c_int, P, P, ctypes.c_int, P, P, ctypes.c_int, ctypes.c_int, ctypes.c_int, P, P]; lib.gaac_read_probe_paged.restype = ctypes.c_int
         _BENCH_LIB = lib
     return _BENCH_LIB
 
@@ -575,6 +576,15 @@ def bench_paged(a):
     sk = torch.empty(cur[li], n_kv, D, dtype=torch.bfloat16, device=dev); sv = torch.empty_like(sk)
     t_dec = _median_us(lambda: st.decode_blocks(buf, pairs, sk, sv), 20)
     dec_bytes = nb_l * 2 * n_kv * 2880 + 2 * sk.numel() * 2
+    # the attention launch's loads without its arithmetic (bench_kernels.hip): same blocks, splits, row order and slot look-ups
+    order = torch.tensor(sorted(range(n_seq), key=lambda i: (-cur[i], i)), dtype=torch.int32, device=dev)
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+    def probe():
+        rc = bench_lib().gaac_read_probe_paged(buf.data_ptr(), st.TS, st.mt.data_ptr(), bt.data_ptr(), bt.stride(0), seq_lens.data_ptr(), order.data_ptr(),
+                                               n_seq, n_kv, nsplit, sink.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        assert rc == 0, rc
+    t_probe = _median_us(probe, 20)
+    t_attn_again = _median_us(lambda: st.attention(q, buf, bt, seq_lens, nsplit, max_seq_len=max_len, out=out_buf), 20)
     # bytes the attention has to read: full slots up to the used escape bytes, raw tiles in full
     mt = st.mt.cpu().numpy().reshape(need_blocks, 2 * n_kv)
     n_tiles = sum(-(-c // BLOCK) for c in cur) * 2 * n_kv
@@ -588,6 +598,8 @@ def bench_paged(a):
     print(json.dumps({"workload": "config 3: paged serving step, 16 sequences, 32 q / 8 kv heads, d=128", "context_tokens": sum(cur), "steps": steps, "nsplit": nsplit,
                       "step_us": round(med(t_step), 1), "step_timing": f"store + attention (which also frees the raw tiles the store gave back) captured once as a HIP graph, replayed per step ({len(t_step)} steps), events around each replay, median",
                       "eager_attention_us": round(med(t_attn), 1), "eager_store_us": round(med(t_store), 1),
+                      "read_probe": {"us": round(t_probe, 1), "attention_timed_the_same_way_us": round(t_attn_again, 1),
+                                     "what": "gaac_read_probe_paged: the attention launch's loads over the same pool without its arithmetic, same blocks, splits and slot look-ups; back-to-back launches, events around each, median"},
                       "attention_read_GBps": round(read_bytes / med(t_attn) / 1e3, 1), "bf16_equivalent_GBps": round(bf16_bytes / med(t_attn) / 1e3, 1),
                       "slot_pool_bytes": pool_bytes, "bf16_pool_bytes": bf16_pool, "pool_ratio": round(bf16_pool / pool_bytes, 4),
                       "raw_tiles_in_use": n_raw, "tiles": n_tiles,
