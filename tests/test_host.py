@@ -44,6 +44,18 @@ def test_ctypes_table_matches_the_header():
         assert _lib._SIGNATURES[name] == want, name
 
 
+def test_every_entry_point_rejects_null_arguments_before_it_touches_a_device():
+    """All-null, all-zero argument lists come back as -1 with a message on the calling thread: the argument checks stand in front
+    of the first HIP call of every entry point.  (The two calls that only take a stream are left out: they do go to the device.)"""
+    from gaac_amd import _lib
+    lib = _lib.load()
+    for name, args in _lib._SIGNATURES.items():
+        if name in ("gaac_static_init", "gaac_static_reset"): continue
+        zeros = [None if a is ctypes.c_void_p else (0.0 if a is ctypes.c_float else 0) for a in args]
+        assert getattr(lib, name)(*zeros) == -1, name
+        assert len(lib.gaac_last_error()) > 8, name
+
+
 def test_no_device_no_fallback():
     """Without a GPU (or with CPU tensors) the product path raises instead of computing on the host."""
     from gaac_amd import Codec
